@@ -1,0 +1,24 @@
+"""Block-sparse attention for AMD MI355X (gfx950): hand-written HIP kernels behind the flex-block-attn operator API."""
+from .interface import (
+    BlockLists,
+    FlexBlockAttnFunc,
+    _flex_block_attn_backward,
+    _flex_block_attn_forward,
+    backward_with_lists,
+    compact_block_mask,
+    flex_block_attn_func,
+    forward_with_lists,
+)
+from . import masks
+
+__all__ = [
+    "flex_block_attn_func",
+    "_flex_block_attn_forward",
+    "_flex_block_attn_backward",
+    "FlexBlockAttnFunc",
+    "BlockLists",
+    "compact_block_mask",
+    "forward_with_lists",
+    "backward_with_lists",
+    "masks",
+]

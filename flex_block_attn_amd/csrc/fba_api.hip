@@ -1,0 +1,179 @@
+// C ABI entry points: argument validation, variant selection, launches.  See include/fba.h for the contract.
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "../../include/fba.h"
+#include "fba_kernels.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+std::atomic<int> g_fwd_qb{0};
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+struct Shape {
+  int64_t mask_bh;
+  int B, Hq, Hkv, Sq, Skv, D, q_block, k_block;
+};
+
+// Shape rules of the operator (flex_block_attn_interface.py:18-32, flex_block_attn_h100.cu:833-850).
+int check_shape(const Shape& s) {
+  if (s.D != 128) return fail(FBA_ERR_INVALID, "head_dim must be 128, got %d", s.D);
+  if (s.B <= 0 || s.Hq <= 0 || s.Hkv <= 0 || s.Sq <= 0 || s.Skv <= 0)
+    return fail(FBA_ERR_INVALID, "B, Hq, Hkv, Sq, Skv must be positive (got %d %d %d %d %d)", s.B, s.Hq, s.Hkv, s.Sq, s.Skv);
+  if (s.Hq % s.Hkv != 0) return fail(FBA_ERR_INVALID, "Hq (%d) must be a multiple of Hkv (%d)", s.Hq, s.Hkv);
+  if (s.q_block <= 0 || s.q_block % 16 != 0) return fail(FBA_ERR_INVALID, "q_block (%d) must be a positive multiple of 16", s.q_block);
+  if (s.k_block <= 0 || s.k_block % 64 != 0) return fail(FBA_ERR_INVALID, "k_block (%d) must be a positive multiple of 64", s.k_block);
+  if (s.k_block % s.q_block != 0 && s.q_block % s.k_block != 0)
+    return fail(FBA_ERR_INVALID, "one of q_block (%d), k_block (%d) must divide the other", s.q_block, s.k_block);
+  if (s.Sq % s.q_block != 0) return fail(FBA_ERR_INVALID, "Sq (%d) must be a multiple of q_block (%d)", s.Sq, s.q_block);
+  if (s.Skv % s.k_block != 0) return fail(FBA_ERR_INVALID, "Skv (%d) must be a multiple of k_block (%d)", s.Skv, s.k_block);
+  if (s.mask_bh != 1 && s.mask_bh != (int64_t)s.B * s.Hq)
+    return fail(FBA_ERR_INVALID, "mask_bh (%lld) must be 1 or B*Hq (%lld)", (long long)s.mask_bh, (long long)s.B * s.Hq);
+  if ((int64_t)s.B * s.Hq * (int64_t)(s.Sq / 128 + 1) > 0x7fffffffLL || (int64_t)s.B * s.Hkv * (int64_t)(s.Skv / 128 + 1) > 0x7fffffffLL)
+    return fail(FBA_ERR_INVALID, "problem too large for a 32-bit work-item index");
+  return FBA_OK;
+}
+
+int check_ptrs(std::initializer_list<std::pair<const char*, const void*>> ps) {
+  for (auto& kv : ps) {
+    if (kv.second == nullptr) return fail(FBA_ERR_INVALID, "%s is null", kv.first);
+    if (!aligned16(kv.second)) return fail(FBA_ERR_INVALID, "%s is not 16-byte aligned", kv.first);
+  }
+  return FBA_OK;
+}
+
+int hip_fail(hipError_t e, const char* what) { return fail(FBA_ERR_HIP, "%s: %s", what, hipGetErrorString(e)); }
+
+}  // namespace
+
+extern "C" {
+
+int32_t fba_version(void) { return 1000; }
+
+const char* fba_last_error(void) { return g_err; }
+
+int32_t fba_set_option(const char* name, int32_t value) {
+  if (name == nullptr) return fail(FBA_ERR_INVALID, "option name is null");
+  if (std::strcmp(name, "fwd_qb") == 0) {
+    if (value < 0 || value > 3) return fail(FBA_ERR_INVALID, "fwd_qb must be 0..3, got %d", value);
+    g_fwd_qb.store(value);
+    return FBA_OK;
+  }
+  return fail(FBA_ERR_INVALID, "unknown option '%s'", name);
+}
+
+int32_t fba_mask_compact(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32_t nK, int32_t* q_cnt, int32_t* q_idx,
+                         int32_t* k_cnt, int32_t* k_idx, void* hip_stream) {
+  if (mask_bh <= 0 || nQ <= 0 || nK <= 0)
+    return fail(FBA_ERR_INVALID, "mask_bh, nQ, nK must be positive (got %lld %d %d)", (long long)mask_bh, nQ, nK);
+  if (!mask || !q_cnt || !q_idx || !k_cnt || !k_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
+  hipError_t e = fba::launch_mask_compact(mask, mask_bh, nQ, nK, q_cnt, q_idx, k_cnt, k_idx, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "mask_compact launch");
+}
+
+int32_t fba_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* q_cnt,
+                const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
+                int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+  const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
+  if (int rc = check_shape(s)) return rc;
+  if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"o", o}})) return rc;
+  if (!lse || !q_cnt || !q_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
+  if (q_block % 128 != 0)
+    return fail(FBA_ERR_UNSUPPORTED, "forward: q_block (%d) must be a multiple of 128 in this build", q_block);
+  int qb = g_fwd_qb.load();
+  if (qb == 0) qb = 1;
+  if (q_block % (128 * qb) != 0) qb = 1;
+
+  fba::FwdParams p{};
+  p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.o = (__bf16*)o; p.lse = lse;
+  p.q_cnt = q_cnt; p.q_idx = q_idx; p.mask_bh = mask_bh;
+  p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Sq = Sq; p.Skv = Skv; p.nQ = Sq / q_block; p.nK = Skv / k_block;
+  p.q_block = q_block; p.k_block = k_block;
+  p.scale_log2e = 1.4426950408889634f / 11.313708498984761f;
+  hipError_t e = fba::launch_fwd(p, qb, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "forward launch");
+}
+
+static int fill_bwd(fba::BwdParams& p, const Shape& s) {
+  p.mask_bh = s.mask_bh;
+  p.B = s.B; p.Hq = s.Hq; p.Hkv = s.Hkv; p.Sq = s.Sq; p.Skv = s.Skv; p.nQ = s.Sq / s.q_block; p.nK = s.Skv / s.k_block;
+  p.q_block = s.q_block; p.k_block = s.k_block;
+  p.scale = 1.f / 11.313708498984761f;
+  p.scale_log2e = 1.4426950408889634f / 11.313708498984761f;
+  return FBA_OK;
+}
+
+int32_t fba_bwd_delta(const void* o, const void* d_o, float* delta, int64_t rows, int32_t head_dim, void* hip_stream) {
+  if (head_dim != 128) return fail(FBA_ERR_INVALID, "head_dim must be 128, got %d", head_dim);
+  if (rows < 0) return fail(FBA_ERR_INVALID, "rows must be non-negative");
+  if (int rc = check_ptrs({{"o", o}, {"d_o", d_o}})) return rc;
+  if (!delta) return fail(FBA_ERR_INVALID, "delta is null");
+  hipError_t e = fba::launch_bwd_delta((const __bf16*)o, (const __bf16*)d_o, delta, rows, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "delta launch");
+}
+
+int32_t fba_bwd_dq(const void* q, const void* k, const void* v, const void* d_o, const float* lse, const float* delta,
+                   void* dq, const int32_t* q_cnt, const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq,
+                   int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,
+                   void* hip_stream) {
+  const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
+  if (int rc = check_shape(s)) return rc;
+  if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"d_o", d_o}, {"dq", dq}})) return rc;
+  if (!lse || !delta || !q_cnt || !q_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
+  if (q_block % 128 != 0)
+    return fail(FBA_ERR_UNSUPPORTED, "dq: q_block (%d) must be a multiple of 128 in this build", q_block);
+  fba::BwdParams p{};
+  fill_bwd(p, s);
+  p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.d_o = (const __bf16*)d_o;
+  p.lse = lse; p.delta = delta; p.dq = (__bf16*)dq; p.q_cnt = q_cnt; p.q_idx = q_idx;
+  hipError_t e = fba::launch_bwd_dq(p, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "dq launch");
+}
+
+int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* lse, const float* delta,
+                     void* dk, void* dv, const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B,
+                     int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block,
+                     int32_t k_block, void* hip_stream) {
+  const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
+  if (int rc = check_shape(s)) return rc;
+  if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"d_o", d_o}, {"dk", dk}, {"dv", dv}})) return rc;
+  if (!lse || !delta || !k_cnt || !k_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
+  if (k_block % 128 != 0)
+    return fail(FBA_ERR_UNSUPPORTED, "dkdv: k_block (%d) must be a multiple of 128 in this build", k_block);
+  if (q_block % 64 != 0)
+    return fail(FBA_ERR_UNSUPPORTED, "dkdv: q_block (%d) must be a multiple of 64 in this build", q_block);
+  fba::BwdParams p{};
+  fill_bwd(p, s);
+  p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.d_o = (const __bf16*)d_o;
+  p.lse = lse; p.delta = delta; p.dk = (__bf16*)dk; p.dv = (__bf16*)dv; p.k_cnt = k_cnt; p.k_idx = k_idx;
+  hipError_t e = fba::launch_bwd_dkdv(p, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "dkdv launch");
+}
+
+int32_t fba_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                float* delta, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
+                const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
+                int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+  const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
+  if (int rc = check_shape(s)) return rc;
+  if (int rc = fba_bwd_delta(o, d_o, delta, (int64_t)B * Hq * Sq, head_dim, hip_stream)) return rc;
+  if (int rc = fba_bwd_dkdv(q, k, v, d_o, lse, delta, dk, dv, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block,
+                            k_block, hip_stream))
+    return rc;
+  return fba_bwd_dq(q, k, v, d_o, lse, delta, dq, q_cnt, q_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block,
+                    hip_stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,153 @@
+// Device-side building blocks shared by the gfx950 attention kernels: vector types, MFMA wrappers, the
+// swizzled LDS tile layout and the operand fetches that go with it.
+//
+// LDS tile layout.  A tile is ROWS x 128 bf16, row-major, 256 bytes per row = 16 chunks of 16 bytes.  Chunk c of
+// row r lives at chunk slot c ^ swz(r), swz(r) = ((r & 3) << 2) | ((r >> 2) & 3).  With 64 four-byte banks:
+//   * a 128-bit row-major operand fetch (16 lanes = 16 consecutive rows, one chunk column) touches 16 distinct
+//     slots, i.e. every bank once;
+//   * a transposing 64-bit fetch (half a wave = 4 consecutive rows x 64 contiguous bytes) lands in 4 distinct
+//     64-byte bank groups, again every bank once;
+//   * the global->LDS copy (16 lanes = one row, 16 chunks) is conflict-free by construction.
+//
+// MFMA 32x32x16 bf16 register layouts (lane = 32*h + i):
+//   A (32 x 16): row i,  k = 8h .. 8h+7          B (16 x 32): col i, k = 8h .. 8h+7
+//   C (32 x 32): col i,  acc[4g + e] is row 8g + 4h + e
+// The A and B layouts are the same function of (lane, k), so an accumulator whose summed index sits in the
+// registers can be re-used, after bf16 packing, as either operand of the next product.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fba {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+#define FBA_LDS __attribute__((address_space(3)))
+#define FBA_DEVICE __device__ __forceinline__
+
+constexpr int kHeadDim = 128;
+constexpr int kRowBytes = kHeadDim * 2;  // one bf16 row of a tile
+constexpr int kWave = 64;
+constexpr int kNumXcd = 8;
+
+FBA_DEVICE int swz(int row) { return ((row & 3) << 2) | ((row >> 2) & 3); }
+
+// byte offset of (row, chunk) inside a swizzled tile
+FBA_DEVICE int tile_off(int row, int chunk) { return row * kRowBytes + ((chunk ^ swz(row)) << 4); }
+
+FBA_DEVICE f32x16 mfma32(bf16x8 a, bf16x8 b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+
+FBA_DEVICE bf16x8 lds_read_b128(const char* base, int off) {
+  return *reinterpret_cast<const bf16x8*>(base + off);
+}
+
+// Transposing 64-bit LDS fetch.  Within each group of 16 lanes, destination lane i receives, as element j,
+// element (i % 4) of the 8 bytes addressed by source lane 4*j + i/4.
+FBA_DEVICE bf16x4 lds_read_tr(const char* base, int off) {
+  return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((FBA_LDS bf16x4*)(base + off));
+}
+
+FBA_DEVICE bf16x8 cat(bf16x4 lo, bf16x4 hi) { return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7); }
+
+// eight fp32 accumulators -> eight bf16 (round to nearest even)
+FBA_DEVICE bf16x8 pack8(float a0, float a1, float a2, float a3, float a4, float a5, float a6, float a7) {
+  bf16x2 p0 = __builtin_convertvector((f32x2){a0, a1}, bf16x2);
+  bf16x2 p1 = __builtin_convertvector((f32x2){a2, a3}, bf16x2);
+  bf16x2 p2 = __builtin_convertvector((f32x2){a4, a5}, bf16x2);
+  bf16x2 p3 = __builtin_convertvector((f32x2){a6, a7}, bf16x2);
+  bf16x4 lo = __builtin_shufflevector(p0, p1, 0, 1, 2, 3);
+  bf16x4 hi = __builtin_shufflevector(p2, p3, 0, 1, 2, 3);
+  return cat(lo, hi);
+}
+
+FBA_DEVICE bf16x4 pack4(float a0, float a1, float a2, float a3) {
+  bf16x2 p0 = __builtin_convertvector((f32x2){a0, a1}, bf16x2);
+  bf16x2 p1 = __builtin_convertvector((f32x2){a2, a3}, bf16x2);
+  return __builtin_shufflevector(p0, p1, 0, 1, 2, 3);
+}
+
+// Exchange between the two half-waves.  v_permlane32_swap a, b exchanges the upper half of a with the lower half of b,
+// so for a = b = x it leaves a = {x.lo, x.lo} and b = {x.hi, x.hi}.  Issued as inline asm: through the compiler builtin
+// with two copies of one value, the two results come back as the same register.  The s_nop covers the wait states the
+// instruction needs after a VALU write of its operands.
+struct HalfPair {
+  float lo, hi;  // value of this lane's row in the lower / upper half-wave
+};
+FBA_DEVICE HalfPair both_halves(float x) {
+  float a = x, b = x;
+  asm("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(a), "+v"(b));
+  return {a, b};
+}
+FBA_DEVICE float max_halves(float x) {
+  const HalfPair p = both_halves(x);
+  return fmaxf(p.lo, p.hi);
+}
+FBA_DEVICE float sum_halves(float x) {
+  const HalfPair p = both_halves(x);
+  return p.lo + p.hi;
+}
+
+FBA_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Work-group id -> logical work item, so that each XCD (work-groups are dealt to the 8 XCDs round-robin) owns one
+// contiguous span of logical items and the items that share K/V (same batch and head) meet in one L2.
+FBA_DEVICE int xcd_remap(int bid, int per_xcd) { return (bid % kNumXcd) * per_xcd + bid / kNumXcd; }
+
+// Cooperative copy of ROWS x 128 bf16 from global (row stride 256 B) into registers, then into a swizzled tile.
+// 256 threads; thread t owns chunk t % 16 of rows t / 16 + 16 i.
+template <int ROWS>
+struct TileCopy {
+  static constexpr int kIters = ROWS / 16;
+  u32x4 reg[kIters];
+  FBA_DEVICE void load(const __bf16* __restrict__ g, int tid) {
+    const char* p = reinterpret_cast<const char*>(g) + (tid >> 4) * kRowBytes + (tid & 15) * 16;
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) reg[i] = *reinterpret_cast<const u32x4*>(p + i * 16 * kRowBytes);
+  }
+  // wr_off = tile_off(tid >> 4, tid & 15), precomputed by the caller
+  FBA_DEVICE void store(char* tile, int wr_off) const {
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) *reinterpret_cast<u32x4*>(tile + wr_off + i * 16 * kRowBytes) = reg[i];
+  }
+};
+
+// Per-lane LDS offsets for row-major A/B operand fetches of a 32-row slab: rd[ks] addresses row (lane % 32),
+// chunk 2*ks + lane/32.  Add 32*kRowBytes per further slab (rows stay congruent mod 16, so swz is unchanged).
+struct RowMajorOffsets {
+  int rd[8];
+  FBA_DEVICE void init(int lane) {
+    const int r = lane & 31, h = lane >> 5;
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) rd[ks] = tile_off(r, 2 * ks + h);
+  }
+};
+
+// Per-lane LDS offsets for transposed operand fetches.  A fetch covers 4 rows (the summed index) x 64 columns...
+// For a 16-wide slice of the summed index starting at row R (R % 16 == 0) and column block cb (32 columns), the lane
+// issues two fetches: rows R + 4h + (lane/4)%4 and the same + 8; columns 32*cb + 16*((lane/16)%2) + 4*(lane%4).
+// The two fetches give k = 8h+0..3 and 8h+4..7 of an operand whose row/col index is 32*cb + lane%32, provided the other
+// operand enumerates the summed index as  R + 8*(t/4) + 4h + t%4  for t = 0..7 (which is exactly the order the 32x32
+// accumulator layout hands its rows out in).
+struct TransposedOffsets {
+  int rd[4][2];  // [column block][+8 rows]
+  FBA_DEVICE void init(int lane) {
+    const int h = lane >> 5;
+    const int rl = 4 * h + ((lane >> 2) & 3);
+    const int cl = 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1);
+    const int inner = (lane & 1) * 8;
+#pragma unroll
+    for (int cb = 0; cb < 4; ++cb) {
+      rd[cb][0] = tile_off(rl, 4 * cb + cl) + inner;
+      rd[cb][1] = tile_off(rl + 8, 4 * cb + cl) + inner;
+    }
+  }
+};
+
+}  // namespace fba

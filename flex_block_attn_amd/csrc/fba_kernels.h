@@ -1,0 +1,56 @@
+// Host-visible parameter blocks and launchers of the gfx950 kernels.  Internal to the shared library; the public
+// surface is the C ABI in include/fba.h.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace fba {
+
+// Active-block lists, as produced by the compaction kernel.
+//   q_cnt [mask_bh, nQ], q_idx [mask_bh, nQ, nK]: for every query block the ascending selected key blocks.
+//   k_cnt [mask_bh, nK], k_idx [mask_bh, nK, nQ]: for every key block the ascending query blocks that select it.
+// mask_bh is B*Hq, or 1 when one 2-D mask is shared by every (batch, head).
+
+struct FwdParams {
+  const __bf16* q;
+  const __bf16* k;
+  const __bf16* v;
+  __bf16* o;
+  float* lse;  // [B, Hq, Sq], natural log
+  const int32_t* q_cnt;
+  const int32_t* q_idx;
+  int64_t mask_bh;
+  int B, Hq, Hkv, Sq, Skv, nQ, nK, q_block, k_block;
+  float scale_log2e;  // log2(e) / sqrt(head_dim)
+  int num_items, items_per_xcd;
+};
+
+struct BwdParams {
+  const __bf16* q;
+  const __bf16* k;
+  const __bf16* v;
+  const __bf16* d_o;
+  const float* lse;
+  const float* delta;  // [B, Hq, Sq]
+  __bf16* dq;
+  __bf16* dk;
+  __bf16* dv;
+  const int32_t* q_cnt;
+  const int32_t* q_idx;
+  const int32_t* k_cnt;
+  const int32_t* k_idx;
+  int64_t mask_bh;
+  int B, Hq, Hkv, Sq, Skv, nQ, nK, q_block, k_block;
+  float scale;        // 1 / sqrt(head_dim)
+  float scale_log2e;  // log2(e) / sqrt(head_dim)
+  int num_items, items_per_xcd;
+};
+
+hipError_t launch_mask_compact(const uint8_t* mask, int64_t mask_bh, int nQ, int nK, int32_t* q_cnt, int32_t* q_idx,
+                               int32_t* k_cnt, int32_t* k_idx, hipStream_t stream);
+hipError_t launch_fwd(FwdParams p, int qb, hipStream_t stream);
+hipError_t launch_bwd_delta(const __bf16* o, const __bf16* d_o, float* delta, int64_t rows, hipStream_t stream);
+hipError_t launch_bwd_dq(BwdParams p, hipStream_t stream);
+hipError_t launch_bwd_dkdv(BwdParams p, hipStream_t stream);
+
+}  // namespace fba

@@ -1,0 +1,85 @@
+// Mask compaction: bool block mask [mask_bh, nQ, nK] -> ascending active-index lists in both orientations.
+//
+// The reference never materialises such lists: every CTA rescans its mask row in the tile loop
+// (flex_block_attn_h100.cu:134-135, :247-248) and the backward pass needs a transposed copy of the mask
+// (flex_block_attn_interface.py:85-86; scan at flex_block_attn_h100.cu:672, :738).  Here one launch emits
+//   q_cnt[m, i], q_idx[m, i, 0..q_cnt) = { j : mask[m, i, j] }   ascending, padded with -1 to nK entries
+//   k_cnt[m, j], k_idx[m, j, 0..k_cnt) = { i : mask[m, i, j] }   ascending, padded with -1 to nQ entries
+// One wave per output row: 64 mask bytes per step, ballot + prefix popcount gives each active lane its slot, so the
+// output order is the index order and the result is independent of scheduling (bit-exact, no atomics).
+#include "fba_common.h"
+#include "fba_kernels.h"
+
+namespace fba {
+
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void mask_compact_kernel(
+    const uint8_t* __restrict__ mask, int64_t mask_bh, int nQ, int nK, int32_t* __restrict__ q_cnt,
+    int32_t* __restrict__ q_idx, int32_t* __restrict__ k_cnt, int32_t* __restrict__ k_idx) {
+  const int lane = threadIdx.x & 63;
+  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t n_qrows = mask_bh * nQ, n_krows = mask_bh * nK;
+  if (w >= n_qrows + n_krows) return;
+
+  const bool row_pass = w < n_qrows;
+  const int64_t r = row_pass ? w : w - n_qrows;
+  const int len = row_pass ? nK : nQ;           // entries per output row
+  const int64_t m = r / (row_pass ? nQ : nK);   // which (batch, head) mask
+  const int self = (int)(r - m * (row_pass ? nQ : nK));
+  const uint8_t* base = mask + m * (int64_t)nQ * nK;
+  // element t of this output row's source: row pass mask[self, t]; column pass mask[t, self]
+  const int64_t stride = row_pass ? 1 : nK;
+  const uint8_t* src = base + (row_pass ? (int64_t)self * nK : (int64_t)self);
+  int32_t* out = (row_pass ? q_idx : k_idx) + r * (int64_t)len;
+
+  int cnt = 0;
+  for (int t0 = 0; t0 < len; t0 += 64) {
+    const int t = t0 + lane;
+    const bool on = t < len && src[(int64_t)t * stride] != 0;
+    const unsigned long long bal = __ballot(on);
+    if (on) out[cnt + __popcll(bal & ((1ull << lane) - 1ull))] = t;
+    cnt += __popcll(bal);
+  }
+  for (int t = cnt + lane; t < len; t += 64) out[t] = -1;
+  if (lane == 0) (row_pass ? q_cnt : k_cnt)[r] = cnt;
+}
+
+hipError_t launch_mask_compact(const uint8_t* mask, int64_t mask_bh, int nQ, int nK, int32_t* q_cnt, int32_t* q_idx,
+                               int32_t* k_cnt, int32_t* k_idx, hipStream_t stream) {
+  const int64_t waves = mask_bh * ((int64_t)nQ + nK);
+  const int64_t blocks = (waves + 3) / 4;
+  if (blocks <= 0) return hipSuccess;
+  if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(mask_compact_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, mask, mask_bh, nQ, nK, q_cnt,
+                     q_idx, k_cnt, k_idx);
+  return hipGetLastError();
+}
+
+// delta[r] = sum_c dO[r, c] * O[r, c] in fp32 (reference: bwd_attend_prep_ker, flex_block_attn_h100.cu:375-379).
+// 16 lanes per row (16 bytes of each operand per lane), 16 rows per 256-thread work-group pass.
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void bwd_delta_kernel(const __bf16* __restrict__ o,
+                                                                                        const __bf16* __restrict__ d_o,
+                                                                                        float* __restrict__ delta, int64_t rows) {
+  const int sub = threadIdx.x & 15;
+  for (int64_t r = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4); r < rows; r += (int64_t)gridDim.x * 16) {
+    const bf16x8 a = *reinterpret_cast<const bf16x8*>(o + r * kHeadDim + sub * 8);
+    const bf16x8 b = *reinterpret_cast<const bf16x8*>(d_o + r * kHeadDim + sub * 8);
+    float acc = 0.f;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) acc += (float)a[t] * (float)b[t];
+    acc += __shfl_xor(acc, 8);
+    acc += __shfl_xor(acc, 4);
+    acc += __shfl_xor(acc, 2);
+    acc += __shfl_xor(acc, 1);
+    if (sub == 0) delta[r] = acc;
+  }
+}
+
+hipError_t launch_bwd_delta(const __bf16* o, const __bf16* d_o, float* delta, int64_t rows, hipStream_t stream) {
+  if (rows <= 0) return hipSuccess;
+  int64_t blocks = (rows + 15) / 16;
+  if (blocks > 65536) blocks = 65536;
+  hipLaunchKernelGGL(bwd_delta_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, o, d_o, delta, rows);
+  return hipGetLastError();
+}
+
+}  // namespace fba

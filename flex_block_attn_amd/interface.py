@@ -1,0 +1,224 @@
+"""Operator surface of flex-block-attn on MI355X.
+
+Same names, argument order and return arity as the reference's flex_block_attn/flex_block_attn_interface.py
+(`flex_block_attn_func` :91-106, `FlexBlockAttnFunc` :14-89, `_flex_block_attn_forward` :6-8,
+`_flex_block_attn_backward` :10-12).  The compiled half is libfba_gfx950.so, reached through ctypes with raw device
+pointers and the current HIP stream; PyTorch only provides device memory and autograd plumbing.
+
+What differs from the reference, deliberately:
+  * the bool block mask is turned into index lists once, on the GPU (`compact_block_mask`), at its true
+    (q_block x kv_block) granularity; the coarse / fine mask pair of flex_block_attn_interface.py:38-66 is not needed;
+  * backward reuses the key-major lists emitted by the same compaction instead of transposing the masks
+    (flex_block_attn_interface.py:85-86);
+  * dq, dk, dv come back in the dtype of q (bf16) rather than fp32 (flex_block_attn_h100.cu:1077-1088);
+  * `lse` is the natural-log softmax denominator, shape (B, H, Sq, 1); the reference's value at that position is
+    -sqrt(128) times it (flex_block_attn_h100.cu:303-307) and is only ever consumed by its own backward.
+"""
+import ctypes
+from dataclasses import dataclass
+
+import torch
+
+from . import _lib
+
+HEAD_DIM = 128
+
+
+@dataclass
+class BlockLists:
+    """Active-block index lists of one block mask (see include/fba.h, fba_mask_compact)."""
+
+    q_cnt: torch.Tensor  # [mask_bh, nQ] int32
+    q_idx: torch.Tensor  # [mask_bh, nQ, nK] int32, ascending, -1 padded
+    k_cnt: torch.Tensor  # [mask_bh, nK] int32
+    k_idx: torch.Tensor  # [mask_bh, nK, nQ] int32, ascending, -1 padded
+    mask_bh: int
+    nQ: int
+    nK: int
+
+    def transposed(self):
+        """Lists of the transposed mask (query and key roles swapped); no device work."""
+        return BlockLists(self.k_cnt, self.k_idx, self.q_cnt, self.q_idx, self.mask_bh, self.nK, self.nQ)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _require_device(t, name):
+    if not t.is_cuda:
+        raise ValueError(f"{name} must be a GPU tensor (the HIP kernels have no CPU fallback)")
+
+
+def compact_block_mask(block_mask):
+    """bool block mask [nQ, nK] or [B, H, nQ, nK] (GPU) -> BlockLists, via the compaction kernel."""
+    if block_mask.dtype != torch.bool:
+        raise TypeError(f"block_mask must be a bool tensor, got {block_mask.dtype}")
+    if block_mask.dim() not in (2, 4):
+        raise ValueError(f"block_mask must have 2 or 4 dimensions, got {block_mask.dim()}")
+    _require_device(block_mask, "block_mask")
+    m = block_mask.contiguous()
+    nQ, nK = m.shape[-2], m.shape[-1]
+    mask_bh = 1 if m.dim() == 2 else m.shape[0] * m.shape[1]
+    dev = m.device
+    q_cnt = torch.empty((mask_bh, nQ), dtype=torch.int32, device=dev)
+    q_idx = torch.empty((mask_bh, nQ, nK), dtype=torch.int32, device=dev)
+    k_cnt = torch.empty((mask_bh, nK), dtype=torch.int32, device=dev)
+    k_idx = torch.empty((mask_bh, nK, nQ), dtype=torch.int32, device=dev)
+    with torch.cuda.device(dev):
+        _lib.call("fba_mask_compact", _ptr(m), mask_bh, nQ, nK, _ptr(q_cnt), _ptr(q_idx), _ptr(k_cnt), _ptr(k_idx), _stream())
+    return BlockLists(q_cnt, q_idx, k_cnt, k_idx, mask_bh, nQ, nK)
+
+
+def _check_qkv(q, k, v):
+    """Tensor contract of the extension (flex_block_attn_h100.cu:820-858)."""
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _require_device(t, name)
+        if t.dtype != torch.bfloat16:
+            raise TypeError(f"{name} must be bfloat16, got {t.dtype}")
+        if t.dim() != 4:
+            raise ValueError(f"{name} must have shape (batch, heads, seq, head_dim)")
+        if not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous")
+    B, Hq, Sq, D = q.shape
+    Bk, Hkv, Skv, Dk = k.shape
+    if D != HEAD_DIM or Dk != HEAD_DIM or v.shape[3] != HEAD_DIM:
+        raise ValueError("head_dim must be 128")
+    if Bk != B or v.shape[0] != B:
+        raise ValueError("q, k, v batch dimensions must match")
+    if v.shape[1] != Hkv or v.shape[2] != Skv:
+        raise ValueError("k and v must have the same shape")
+    if Hq % Hkv != 0:
+        raise ValueError("q heads must be a multiple of kv heads")
+    return B, Hq, Hkv, Sq, Skv
+
+
+def _check_blocks(q, k, q_block_size, kv_block_size, block_mask):
+    """Block-size and mask-shape rules (flex_block_attn_interface.py:18-32)."""
+    assert q_block_size % 16 == 0, f"q_block_size ({q_block_size}) must be divisible by 16"
+    assert kv_block_size % 64 == 0, f"kv_block_size ({kv_block_size}) must be divisible by 64"
+    assert kv_block_size % q_block_size == 0 or q_block_size % kv_block_size == 0, (
+        f"kv_block_size ({kv_block_size}) must be divisible by q_block_size ({q_block_size}), or vice versa."
+    )
+    q_seq_len, kv_seq_len = q.shape[2], k.shape[2]
+    assert q_seq_len % q_block_size == 0, f"q_seq_len ({q_seq_len}) must be divisible by q_block_size ({q_block_size})"
+    assert kv_seq_len % kv_block_size == 0, f"kv_seq_len ({kv_seq_len}) must be divisible by kv_block_size ({kv_block_size})"
+    if block_mask.dim() not in (2, 4):
+        raise ValueError(f"block_mask must have 2 or 4 dimensions, got {block_mask.dim()}")
+    q_block_num, kv_block_num = block_mask.shape[-2], block_mask.shape[-1]
+    assert q_block_size * q_block_num == q_seq_len, (
+        f"q_block_size ({q_block_size}) * q_block_num ({q_block_num}) must equal q_seq_len ({q_seq_len})"
+    )
+    assert kv_block_size * kv_block_num == kv_seq_len, (
+        f"kv_block_size ({kv_block_size}) * kv_block_num ({kv_block_num}) must equal kv_seq_len ({kv_seq_len})"
+    )
+    if block_mask.dim() == 4 and tuple(block_mask.shape[:2]) != (q.shape[0], q.shape[1]):
+        raise ValueError(
+            f"4-D block_mask must be [batch, heads, q_blocks, kv_blocks] = [{q.shape[0]}, {q.shape[1]}, ...], "
+            f"got {tuple(block_mask.shape)}"
+        )
+
+
+def _check_lists(lists, B, Hq, Sq, Skv, q_block_size, kv_block_size):
+    if lists.nQ * q_block_size != Sq or lists.nK * kv_block_size != Skv:
+        raise ValueError("block lists do not match the sequence lengths and block sizes")
+    if lists.mask_bh not in (1, B * Hq):
+        raise ValueError("block lists do not match batch * heads")
+
+
+def forward_with_lists(q, k, v, q_block_size, kv_block_size, lists):
+    """Forward on compacted lists -> (o [B,H,Sq,128] bf16, lse [B,H,Sq,1] fp32)."""
+    B, Hq, Hkv, Sq, Skv = _check_qkv(q, k, v)
+    _check_lists(lists, B, Hq, Sq, Skv, q_block_size, kv_block_size)
+    o = torch.empty_like(q)
+    lse = torch.empty((B, Hq, Sq, 1), dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        _lib.call(
+            "fba_fwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(lists.q_cnt), _ptr(lists.q_idx), lists.mask_bh,
+            B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size, _stream(),
+        )
+    return o, lse
+
+
+def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists):
+    """Backward on compacted lists -> (dq, dk, dv), bf16, shaped like q, k, v."""
+    B, Hq, Hkv, Sq, Skv = _check_qkv(q, k, v)
+    _check_lists(lists, B, Hq, Sq, Skv, q_block_size, kv_block_size)
+    if do.dtype != torch.bfloat16:
+        do = do.to(torch.bfloat16)
+    do = do.contiguous()
+    o = o.contiguous()
+    if o.shape != q.shape or do.shape != q.shape:
+        raise ValueError("o and do must have the shape of q")
+    if lse.dtype != torch.float32 or lse.numel() != B * Hq * Sq:
+        raise ValueError("lse must be float32 with B*H*Sq elements")
+    lse = lse.contiguous()
+    dq = torch.empty_like(q)
+    dk = torch.empty_like(k)
+    dv = torch.empty_like(v)
+    delta = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        _lib.call(
+            "fba_bwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(delta), _ptr(dq), _ptr(dk), _ptr(dv),
+            _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), lists.mask_bh,
+            B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size, _stream(),
+        )
+    return dq, dk, dv
+
+
+def _flex_block_attn_forward(q, k, v, q_block_size, kv_block_size, block_mask, small_block_mask, use_small_block_mode):
+    """Drop-in for flex_block_attn_interface.py:6-8.  `small_block_mask` is the mask at (q_block x kv_block)
+    granularity (it equals `block_mask` when the two block sizes agree); `block_mask`, the max-pooled copy the
+    reference's kernel needs, is accepted and ignored."""
+    fine = small_block_mask if use_small_block_mode else block_mask
+    _check_blocks(q, k, q_block_size, kv_block_size, fine)
+    lists = compact_block_mask(fine)
+    return forward_with_lists(q, k, v, q_block_size, kv_block_size, lists)
+
+
+def _flex_block_attn_backward(q, k, v, o, lse, do, q_block_size, kv_block_size, block_mask, small_block_mask, use_small_block_mode):
+    """Drop-in for flex_block_attn_interface.py:10-12.  As in the reference, both masks arrive TRANSPOSED
+    ([..., kv_blocks, q_blocks], flex_block_attn_interface.py:85-86)."""
+    fine_t = small_block_mask if use_small_block_mode else block_mask
+    if fine_t.dim() not in (2, 4):
+        raise ValueError(f"block_mask must have 2 or 4 dimensions, got {fine_t.dim()}")
+    lists = compact_block_mask(fine_t).transposed()
+    return backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists)
+
+
+class FlexBlockAttnFunc(torch.autograd.Function):
+    """autograd wrapper, same signature as flex_block_attn_interface.py:14-89."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, q_block_size, kv_block_size, block_mask, is_grad_enabled):
+        _check_blocks(q, k, q_block_size, kv_block_size, block_mask)
+        is_grad = is_grad_enabled and any(x.requires_grad for x in [q, k, v])
+        lists = compact_block_mask(block_mask)
+        o, lse = forward_with_lists(q, k, v, q_block_size, kv_block_size, lists)
+        if is_grad:
+            ctx.save_for_backward(q, k, v, o, lse, lists.q_cnt, lists.q_idx, lists.k_cnt, lists.k_idx)
+            ctx.q_block_size = q_block_size
+            ctx.kv_block_size = kv_block_size
+            ctx.list_meta = (lists.mask_bh, lists.nQ, lists.nK)
+        return o
+
+    @staticmethod
+    def backward(ctx, dout, *args):
+        q, k, v, o, lse, q_cnt, q_idx, k_cnt, k_idx = ctx.saved_tensors
+        lists = BlockLists(q_cnt, q_idx, k_cnt, k_idx, *ctx.list_meta)
+        dq, dk, dv = backward_with_lists(q, k, v, o, lse, dout, ctx.q_block_size, ctx.kv_block_size, lists)
+        return dq, dk, dv, None, None, None, None
+
+
+def flex_block_attn_func(q, k, v, q_block_size, kv_block_size, block_mask):
+    """Block-sparse attention: softmax(q k^T / sqrt(128)) v restricted, per query block, to the key blocks that
+    `block_mask` selects.
+
+    q: (batch, heads, q_seq_len, 128) bf16; k, v: (batch, kv_heads, kv_seq_len, 128) bf16; block_mask: bool
+    [q_seq_len / q_block_size, kv_seq_len / kv_block_size] or [batch, heads, ...]. Returns o shaped like q.
+    """
+    return FlexBlockAttnFunc.apply(q, k, v, q_block_size, kv_block_size, block_mask, torch.is_grad_enabled())

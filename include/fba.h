@@ -1,0 +1,98 @@
+/*
+ * C ABI of the gfx950 block-sparse attention library (libfba_gfx950.so).
+ *
+ * The library replaces the compiled half of the reference operator: the pybind11 module `flex_block_attn_cuda`
+ * (attn.cpp:25-31) with its two entry points attn_forward / attn_backward, whose host launchers live at
+ * flex_block_attn/flex_block_attn_h100.cu:810-1007 and :1009-1267.  Differences in contract:
+ *   - plain pointers and sizes, no torch types; the caller owns every buffer (the reference allocates its outputs
+ *     with torch::empty / torch::zeros, flex_block_attn_h100.cu:865-874, :1077-1093);
+ *   - everything is enqueued on the HIP stream passed in and nothing synchronises the device (the reference brackets
+ *     every launch with cudaDeviceSynchronize, :882, :1004-1005, :1113, :1212-1213);
+ *   - the block mask is consumed as compacted index lists produced by fba_mask_compact rather than rescanned by
+ *     every work-group (:134-135, :247-248, :672, :738); the transposed lists replace the transposed mask copies of
+ *     flex_block_attn/flex_block_attn_interface.py:85-86;
+ *   - gradients are written as bf16 directly (the reference returns fp32 buffers filled by reducing stores).
+ *
+ * Tensor layout, as in the reference (flex_block_attn_h100.cu:820-858): q [B, Hq, Sq, 128], k and v
+ * [B, Hkv, Skv, 128], o like q; bf16, contiguous, 16-byte aligned.  lse and delta are fp32 [B, Hq, Sq].
+ * Hq must be a multiple of Hkv (:843-844); kv head = q head / (Hq / Hkv).
+ *
+ * Every function returns FBA_OK or an error code; fba_last_error() gives the message of the calling thread's last
+ * failure.  No function throws or aborts.
+ */
+#ifndef FBA_H_
+#define FBA_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FBA_OK 0
+#define FBA_ERR_INVALID 1     /* an argument violates the contract (shape, alignment, null pointer) */
+#define FBA_ERR_UNSUPPORTED 2 /* valid for the operator, but no kernel variant covers it yet */
+#define FBA_ERR_HIP 3         /* a HIP runtime call failed */
+
+/* Library version: major * 1000 + minor. */
+int32_t fba_version(void);
+
+/* Message for the last non-OK return on the calling thread ("" if none). The pointer stays valid until the next
+ * failing call on the same thread. */
+const char* fba_last_error(void);
+
+/*
+ * Mask compaction.  Replaces the per-CTA mask scans of flex_block_attn_h100.cu:110, :134, :171, :247 (forward) and
+ * :645, :672, :703, :738, :780 (backward, on the transposed mask).
+ *   mask     [mask_bh, nQ, nK] bytes, non-zero = selected; mask_bh = B*Hq, or 1 for one mask shared by all (b, h)
+ *   q_cnt    [mask_bh, nQ]        number of selected key blocks of each query block
+ *   q_idx    [mask_bh, nQ, nK]    their indices, ascending, padded with -1
+ *   k_cnt    [mask_bh, nK]        number of query blocks selecting each key block
+ *   k_idx    [mask_bh, nK, nQ]    their indices, ascending, padded with -1
+ */
+int32_t fba_mask_compact(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32_t nK, int32_t* q_cnt, int32_t* q_idx,
+                         int32_t* k_cnt, int32_t* k_idx, void* hip_stream);
+
+/*
+ * Forward.  Replaces attn_forward (attn.cpp:29, flex_block_attn_h100.cu:810-1007; kernel :52-318).
+ * Writes o (bf16) and lse (fp32, natural log of the row's softmax denominator including the 1/sqrt(128) scale;
+ * -inf and o = 0 for a query block with an empty list).  nQ = Sq / q_block, nK = Skv / k_block.
+ */
+int32_t fba_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* q_cnt,
+                const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
+                int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+
+/*
+ * Backward, three stream-ordered launches.  Replaces attn_backward (attn.cpp:30,
+ * flex_block_attn_h100.cu:1009-1267): bwd_attend_prep_ker (:324-389) and bwd_attend_ker (:572-802).
+ *   delta    [B, Hq, Sq] fp32 workspace, written by the call (rowsum(dO o O))
+ *   dq       [B, Hq, Sq, 128] bf16;  dk, dv [B, Hkv, Skv, 128] bf16 (summed over the query heads of a GQA group)
+ * Every output element is written exactly once; no buffer needs clearing beforehand.
+ */
+int32_t fba_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                float* delta, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
+                const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
+                int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+
+/* The three stages of fba_bwd, separately (same arguments, for profiling one kernel at a time). */
+int32_t fba_bwd_delta(const void* o, const void* d_o, float* delta, int64_t rows, int32_t head_dim, void* hip_stream);
+int32_t fba_bwd_dq(const void* q, const void* k, const void* v, const void* d_o, const float* lse, const float* delta,
+                   void* dq, const int32_t* q_cnt, const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq,
+                   int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,
+                   void* hip_stream);
+int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* lse, const float* delta,
+                     void* dk, void* dv, const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B,
+                     int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block,
+                     int32_t k_block, void* hip_stream);
+
+/*
+ * Tuning knobs for experiments (process-wide).  Known names: "fwd_qb" (query rows per forward work-group in units
+ * of 128; 0 = choose automatically).  Returns FBA_ERR_INVALID for an unknown name or value.
+ */
+int32_t fba_set_option(const char* name, int32_t value);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* FBA_H_ */

@@ -1,0 +1,237 @@
+"""CPU oracle for the block-sparse attention operator — TEST INFRASTRUCTURE ONLY.
+
+Nothing in the product imports this module: only tests/, `__graft_entry__.smoke()` and the `cpu_baseline` leg of
+bench.py may.  It restates the reference's dense path in three independent ways so that each can check the others:
+
+  * `dense_attention_explicit`  the textbook formula written out with matmul / exp / sum in fp32 or fp64, plus
+    closed-form gradients (`dense_attention_backward_explicit`);
+  * `sdpa_dense`                the library routine the reference itself uses as its dense path,
+    `F.scaled_dot_product_attention(q, k, v, attn_mask=dense bool mask)` (test/test_flex_block_attn.py:48-51,
+    benchmark/utils/utils.py:132-138), with gradients from autograd;
+  * the plain-C restatement in attn_ref.c (double accumulation, OpenMP), reached through `c_*` wrappers.
+
+Semantics restated (reference file:line):
+  allowed(i, j) = block_mask[b, h, i // q_block, j // kv_block]          benchmark/utils/utils.py:105-119
+  O = softmax(Q K^T / sqrt(128) | allowed) V                             flex_block_attn_h100.cu:177, :199-221, :292
+  delta = rowsum(dO o O)                                                 flex_block_attn_h100.cu:375-379
+  P = exp(S/sqrt(D) - LSE); dV = P^T dO; dP = dO V^T;
+  dS = P o (dP - delta)/sqrt(D); dQ = dS K; dK = dS^T Q                  flex_block_attn_h100.cu:498-537, :750-753
+  kv head of q head h = h // (Hq / Hkv); dK, dV summed over the group    flex_block_attn_h100.cu:80, :615, :555-556
+  work lists = ascending nonzero indices per mask row / column           flex_block_attn_h100.cu:134-135, :672
+
+Parity status: O and LSE are pinned by SDPA, by the explicit formula, by special cases and by brute force
+(tests/test_oracle.py).  dQ, dK, dV have no assertion anywhere in the reference (its dQ check is commented out,
+test/test_flex_block_attn.py:140, and its benchmark comparison is vacuous); they are pinned here by autograd of
+SDPA, by the closed form and by fp64 finite differences.
+"""
+import ctypes
+import math
+import os
+
+import numpy as np
+import torch
+import torch.nn.functional as F
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+C_LIB_PATH = os.path.join(_HERE, "libattn_ref.so")
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# masks and work lists
+# ---------------------------------------------------------------------------------------------------------------
+def expand_block_mask(block_mask, q_block, kv_block):
+    """[..., nQ, nK] bool -> [..., nQ*q_block, nK*kv_block] bool (benchmark/utils/utils.py:105-119)."""
+    return block_mask.repeat_interleave(q_block, dim=-2).repeat_interleave(kv_block, dim=-1)
+
+
+def compact_lists(block_mask):
+    """Work lists of a bool mask [nQ, nK] or [B, H, nQ, nK] by brute force on the host.
+
+    Returns int32 numpy arrays (q_cnt [M,nQ], q_idx [M,nQ,nK], k_cnt [M,nK], k_idx [M,nK,nQ]), M = B*H or 1;
+    lists ascending, padded with -1.
+    """
+    m = block_mask.detach().cpu().numpy().astype(bool)
+    nQ, nK = m.shape[-2:]
+    m = m.reshape(-1, nQ, nK)
+    M = m.shape[0]
+    q_cnt = np.zeros((M, nQ), np.int32)
+    q_idx = np.full((M, nQ, nK), -1, np.int32)
+    k_cnt = np.zeros((M, nK), np.int32)
+    k_idx = np.full((M, nK, nQ), -1, np.int32)
+    for b in range(M):
+        for i in range(nQ):
+            js = np.nonzero(m[b, i])[0]
+            q_cnt[b, i] = len(js)
+            q_idx[b, i, : len(js)] = js
+        for j in range(nK):
+            is_ = np.nonzero(m[b, :, j])[0]
+            k_cnt[b, j] = len(is_)
+            k_idx[b, j, : len(is_)] = is_
+    return q_cnt, q_idx, k_cnt, k_idx
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# restatement 1: explicit formula
+# ---------------------------------------------------------------------------------------------------------------
+def _broadcast_kv(x, Hq):
+    """[B, Hkv, S, D] -> [B, Hq, S, D], q head h reading kv head h // (Hq / Hkv)."""
+    Hkv = x.shape[1]
+    return x if Hkv == Hq else x.repeat_interleave(Hq // Hkv, dim=1)
+
+
+def dense_attention_explicit(q, k, v, block_mask, q_block, kv_block, dtype=torch.float32):
+    """Returns (o, lse) in `dtype`; rows with no allowed key give o = 0, lse = -inf."""
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    Hq, D = q.shape[1], q.shape[3]
+    kk, vv = _broadcast_kv(k, Hq), _broadcast_kv(v, Hq)
+    allowed = expand_block_mask(block_mask.to(q.device), q_block, kv_block)
+    s = torch.matmul(q, kk.transpose(-1, -2)) / math.sqrt(D)
+    s = s.masked_fill(~allowed, float("-inf"))
+    lse = torch.logsumexp(s, dim=-1)
+    p = torch.exp(s - lse.unsqueeze(-1).clamp_min(torch.finfo(dtype).min))
+    p = torch.where(torch.isfinite(lse).unsqueeze(-1), p, torch.zeros_like(p))
+    return torch.matmul(p, vv), lse
+
+
+def dense_attention_backward_explicit(q, k, v, o, lse, do, block_mask, q_block, kv_block, dtype=torch.float32):
+    """Closed-form gradients (dq, dk, dv) in `dtype`."""
+    q, k, v, o, lse, do = (t.to(dtype) for t in (q, k, v, o, lse, do))
+    B, Hq, Sq, D = q.shape
+    Hkv, Skv = k.shape[1], k.shape[2]
+    kk, vv = _broadcast_kv(k, Hq), _broadcast_kv(v, Hq)
+    allowed = expand_block_mask(block_mask.to(q.device), q_block, kv_block)
+    s = torch.matmul(q, kk.transpose(-1, -2)) / math.sqrt(D)
+    p = torch.exp(s - lse.reshape(B, Hq, Sq, 1))
+    p = torch.where(allowed & torch.isfinite(lse.reshape(B, Hq, Sq, 1)), p, torch.zeros_like(p))
+    delta = (do * o).sum(-1, keepdim=True)
+    dv = torch.matmul(p.transpose(-1, -2), do)
+    dp = torch.matmul(do, vv.transpose(-1, -2))
+    ds = p * (dp - delta) / math.sqrt(D)
+    dq = torch.matmul(ds, kk)
+    dk = torch.matmul(ds.transpose(-1, -2), q)
+    if Hkv != Hq:
+        g = Hq // Hkv
+        dk = dk.reshape(B, Hkv, g, Skv, D).sum(2)
+        dv = dv.reshape(B, Hkv, g, Skv, D).sum(2)
+    return dq, dk, dv
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# restatement 2: the library routine the reference calls
+# ---------------------------------------------------------------------------------------------------------------
+def sdpa_dense(q, k, v, block_mask, q_block, kv_block, do=None):
+    """F.scaled_dot_product_attention on the expanded mask, in the dtype of q.  With `do`, also returns
+    (dq, dk, dv) from autograd."""
+    Hq = q.shape[1]
+    allowed = expand_block_mask(block_mask.to(q.device), q_block, kv_block)
+    if do is None:
+        return F.scaled_dot_product_attention(q, _broadcast_kv(k, Hq), _broadcast_kv(v, Hq), attn_mask=allowed)
+    q_, k_, v_ = (t.detach().clone().requires_grad_(True) for t in (q, k, v))
+    o = F.scaled_dot_product_attention(q_, _broadcast_kv(k_, Hq), _broadcast_kv(v_, Hq), attn_mask=allowed)
+    o.backward(do)
+    return o.detach(), q_.grad, k_.grad, v_.grad
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# restatement 3: plain C (attn_ref.c)
+# ---------------------------------------------------------------------------------------------------------------
+_clib = None
+
+
+def c_lib():
+    global _clib
+    if _clib is None:
+        if not os.path.exists(C_LIB_PATH):
+            raise ImportError(f"{C_LIB_PATH} missing: run `python oracle/build_oracle.py`")
+        lib = ctypes.CDLL(C_LIB_PATH)
+        P, I, L = ctypes.c_void_p, ctypes.c_int, ctypes.c_int64
+        lib.oracle_num_threads.restype = I
+        lib.oracle_set_num_threads.argtypes = [I]
+        lib.oracle_expand_block_mask.argtypes = [P, I, I, I, I, P]
+        lib.oracle_mask_compact.argtypes = [P, L, I, I, P, P, P, P]
+        lib.oracle_attn_fwd.argtypes = [P, P, P, P, L, I, I, I, I, I, I, I, I, P, P]
+        lib.oracle_bwd_delta.argtypes = [P, P, L, I, P]
+        lib.oracle_attn_bwd.argtypes = [P, P, P, P, P, P, P, L, I, I, I, I, I, I, I, I, P, P, P]
+        _clib = lib
+    return _clib
+
+
+def _f32(t):
+    return np.ascontiguousarray(t.detach().cpu().to(torch.float32).numpy())
+
+
+def _u8(t):
+    return np.ascontiguousarray(t.detach().cpu().numpy().astype(np.uint8))
+
+
+def _p(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def c_compact_lists(block_mask):
+    m = _u8(block_mask)
+    nQ, nK = m.shape[-2:]
+    M = 1 if m.ndim == 2 else m.shape[0] * m.shape[1]
+    q_cnt = np.empty((M, nQ), np.int32)
+    q_idx = np.empty((M, nQ, nK), np.int32)
+    k_cnt = np.empty((M, nK), np.int32)
+    k_idx = np.empty((M, nK, nQ), np.int32)
+    c_lib().oracle_mask_compact(_p(m), M, nQ, nK, _p(q_cnt), _p(q_idx), _p(k_cnt), _p(k_idx))
+    return q_cnt, q_idx, k_cnt, k_idx
+
+
+def c_expand_block_mask(block_mask, q_block, kv_block):
+    m = _u8(block_mask)
+    nQ, nK = m.shape
+    out = np.empty((nQ * q_block, nK * kv_block), np.uint8)
+    c_lib().oracle_expand_block_mask(_p(m), nQ, nK, q_block, kv_block, _p(out))
+    return torch.from_numpy(out.astype(bool))
+
+
+def c_attention_forward(q, k, v, block_mask, q_block, kv_block):
+    """fp32 (o, lse) from attn_ref.c."""
+    qa, ka, va, m = _f32(q), _f32(k), _f32(v), _u8(block_mask)
+    B, Hq, Sq, D = qa.shape
+    Hkv, Skv = ka.shape[1], ka.shape[2]
+    M = 1 if m.ndim == 2 else B * Hq
+    o = np.empty_like(qa)
+    lse = np.empty((B, Hq, Sq), np.float32)
+    c_lib().oracle_attn_fwd(_p(qa), _p(ka), _p(va), _p(m), M, B, Hq, Hkv, Sq, Skv, D, q_block, kv_block, _p(o), _p(lse))
+    return torch.from_numpy(o), torch.from_numpy(lse)
+
+
+def c_attention_backward(q, k, v, o, lse, do, block_mask, q_block, kv_block):
+    """fp32 (dq, dk, dv) from attn_ref.c."""
+    qa, ka, va, oa, la, da, m = _f32(q), _f32(k), _f32(v), _f32(o), _f32(lse), _f32(do), _u8(block_mask)
+    B, Hq, Sq, D = qa.shape
+    Hkv, Skv = ka.shape[1], ka.shape[2]
+    M = 1 if m.ndim == 2 else B * Hq
+    dq, dk, dv = np.empty_like(qa), np.empty_like(ka), np.empty_like(va)
+    c_lib().oracle_attn_bwd(
+        _p(qa), _p(ka), _p(va), _p(oa), _p(la), _p(da), _p(m), M, B, Hq, Hkv, Sq, Skv, D, q_block, kv_block, _p(dq), _p(dk), _p(dv)
+    )
+    return torch.from_numpy(dq), torch.from_numpy(dk), torch.from_numpy(dv)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# shared helpers for parity tests
+# ---------------------------------------------------------------------------------------------------------------
+def seeded_qkv(B, Hq, Hkv, Sq, Skv, D=128, seed=0, peaky=False):
+    """fp32 q, k, v, do from a CPU generator.  `peaky` reproduces the reference test's input distribution: a random
+    direction times a N(0.1, 10) magnitude per row (test/test_flex_block_attn.py:58-64)."""
+    g = torch.Generator(device="cpu").manual_seed(seed)
+
+    def draw(shape):
+        t = torch.randn(shape, generator=g)
+        if peaky:
+            mag = torch.randn(shape[:-1] + (1,), generator=g) * 10.0 + 0.1
+            t = t * mag / t.norm(dim=-1, keepdim=True)
+        return t
+
+    return draw((B, Hq, Sq, D)), draw((B, Hkv, Skv, D)), draw((B, Hkv, Skv, D)), torch.randn((B, Hq, Sq, D), generator=g)
+
+
+def error_metrics(got, ref):
+    """(max-abs error, relative L2 error) of `got` against `ref`, computed in fp64."""
+    g, r = got.detach().double().cpu(), ref.detach().double().cpu()
+    return (g - r).abs().max().item(), ((g - r).norm() / r.norm().clamp_min(1e-30)).item()
