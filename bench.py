@@ -1,0 +1,217 @@
+#!/usr/bin/env python3
+"""Benchmark of the block-sparse attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload random|full|sta|ssta] [--no-cpu]
+
+One step = mask compaction + forward + backward (delta, dK/dV, dQ) on synthetic inputs already resident in HBM.
+Default workload: B=1, H=24, S=30720, head_dim 128, bf16, 384-token blocks (80x80), an independent random mask per
+(batch, head) keeping 32 of 80 key blocks per query-block row with the diagonal forced on.
+FLOPs count selected block pairs only: forward 4*Bq*Bk*D, backward 10*Bq*Bk*D per pair.
+Prints ONE JSON line on stdout (everything else goes to stderr).
+"""
+import argparse
+import ctypes
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0
+D = 128
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def build_workload(name, device):
+    from flex_block_attn_amd import masks
+
+    if name == "random":
+        B, H, S, qbs, kbs = 1, 24, 30720, 384, 384
+        mask = masks.random_block_mask(B, H, S // qbs, S // kbs, 32, seed=0)
+        desc = "dynamic random sparse: B1 H24 S30720 D128 bf16, block 384 (80x80), per-(b,h) mask, 32 of 80 key blocks kept per row (sparsity 0.6), diagonal on"
+    elif name == "full":
+        B, H, S, qbs, kbs = 1, 24, 11520, 384, 384
+        mask = masks.full_block_mask(S // qbs, S // kbs)
+        desc = "full attention: B1 H24 S11520 D128 bf16, block 384 (30x30), all-ones 2-D mask"
+    elif name == "sta":
+        B, H, S, qbs, kbs = 1, 24, 115200, 384, 384
+        mask = masks.sta_3d_block_mask((5, 6, 10), (3, 3, 3), clamp=True)
+        desc = "3-D sliding-tile mask: B1 H24 S115200 D128 bf16, 300 tiles of 6x8x8=384 tokens, 3x3x3 tile window (clamped), 2-D mask"
+    elif name == "ssta":
+        raise SystemExit("workload 'ssta' needs the GPU mask builder, which this build does not have yet")
+    else:
+        raise SystemExit(f"unknown workload {name}")
+    g = torch.Generator(device="cpu").manual_seed(1234)
+    shape = (B, H, S, D)
+    q, k, v, do = (torch.randn(shape, generator=g, dtype=torch.float32).to(torch.bfloat16).to(device) for _ in range(4))
+    return dict(B=B, H=H, S=S, qbs=qbs, kbs=kbs, mask=mask.to(device), q=q, k=k, v=v, do=do, desc=desc, nnz=int(mask.sum().item()) * (1 if mask.dim() == 4 else B * H))
+
+
+def time_events(fn, warmup, iters):
+    """Per-call durations (ms) of fn on torch's current stream, from HIP events around each call."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for a, b in evs:
+        a.record()
+        fn()
+        b.record()
+    torch.cuda.synchronize()
+    return [a.elapsed_time(b) for a, b in evs]
+
+
+def cpu_baseline(seconds_budget=12.0):
+    """The reference's CPU path (dense-mask scaled_dot_product_attention + backward, fp32) as restated by the oracle,
+    on this machine's host cores: B1 H2 S1536 D128, 4x4 Bernoulli(0.5) block mask with the diagonal on."""
+    from oracle import attn_oracle
+    from flex_block_attn_amd import masks
+
+    cores = os.cpu_count() or 1
+    threads = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(threads)
+    B, H, S, bs = 1, 2, 1536, 384
+    q, k, v, do = attn_oracle.seeded_qkv(B, H, H, S, S, seed=0)
+    mask = masks.bernoulli_block_mask(S // bs, S // bs, 0.5, 0)
+    attn_oracle.sdpa_dense(q, k, v, mask, bs, bs, do)  # warm-up
+    times = []
+    t_end = time.perf_counter() + seconds_budget
+    while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 200):
+        t0 = time.perf_counter()
+        attn_oracle.sdpa_dense(q, k, v, mask, bs, bs, do)
+        times.append(time.perf_counter() - t0)
+    med = statistics.median(times)
+    dense_flops = 14.0 * S * S * D * H * B
+    return {
+        "value": dense_flops / med * 1e-12,
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"oracle sdpa_dense fwd+bwd fp32, B1 H2 S1536 D128 block 384 dense-expanded 4x4 mask, dense FLOPs 14*S^2*D*H, median of {len(times)} runs ({med * 1e3:.1f} ms each), host has {cores} cpus",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="random")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--fwd-qb", type=int, default=0, help="tuning: forward work-group height in units of 128 rows")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py measures one GPU only: every box in this build has a single MI355X (use --gpus 1)")
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+
+    import flex_block_attn_amd as fba
+    from flex_block_attn_amd import _lib
+    from flex_block_attn_amd.interface import _ptr, _stream
+
+    _lib.load()
+    if args.fwd_qb:
+        _lib.call("fba_set_option", b"fwd_qb", args.fwd_qb)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    w = build_workload(args.workload, dev)
+    B, H, S, qbs, kbs = w["B"], w["H"], w["S"], w["qbs"], w["kbs"]
+    q, k, v, do, mask = w["q"], w["k"], w["v"], w["do"], w["mask"]
+    nnz = w["nnz"]
+    pair_flops = float(qbs) * kbs * D
+    fl_fwd, fl_bwd = 4.0 * pair_flops * nnz, 10.0 * pair_flops * nnz
+    log(f"workload: {w['desc']}; nnz block pairs = {nnz}; fwd {fl_fwd * 1e-12:.3f} TFLOP, bwd {fl_bwd * 1e-12:.3f} TFLOP")
+
+    def step():
+        lists = fba.compact_block_mask(mask)
+        o, lse = fba.forward_with_lists(q, k, v, qbs, kbs, lists)
+        return fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists)
+
+    # ---- whole-step timing (the contract's K timed steps) -------------------------------------------------
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = (fl_fwd + fl_bwd) / (ms_per_step * 1e-3) * 1e-12
+
+    # ---- per-kernel timing with HIP events on the launch stream -------------------------------------------
+    lists = fba.compact_block_mask(mask)
+    o, lse = fba.forward_with_lists(q, k, v, qbs, kbs, lists)
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    delta = torch.empty((B, H, S), dtype=torch.float32, device=dev)
+    o2, lse2 = torch.empty_like(o), torch.empty_like(lse)
+    common = (lists.mask_bh, B, H, H, S, S, D, qbs, kbs)
+    kernels = {
+        "mask_compact": lambda: _lib.call("fba_mask_compact", _ptr(mask), lists.mask_bh, lists.nQ, lists.nK, _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), _stream()),
+        "fwd": lambda: _lib.call("fba_fwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o2), _ptr(lse2), _ptr(lists.q_cnt), _ptr(lists.q_idx), *common, _stream()),
+        "bwd_delta": lambda: _lib.call("fba_bwd_delta", _ptr(o), _ptr(do), _ptr(delta), B * H * S, D, _stream()),
+        "bwd_dkdv": lambda: _lib.call("fba_bwd_dkdv", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(lse), _ptr(delta), _ptr(dk), _ptr(dv), _ptr(lists.k_cnt), _ptr(lists.k_idx), *common, _stream()),
+        "bwd_dq": lambda: _lib.call("fba_bwd_dq", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(lse), _ptr(delta), _ptr(dq), _ptr(lists.q_cnt), _ptr(lists.q_idx), *common, _stream()),
+    }
+    iters = max(5, args.steps)
+    kms = {}
+    for name, fn in kernels.items():
+        ts = time_events(fn, max(2, args.warmup), iters)
+        kms[name] = {"mean_ms": sum(ts) / len(ts), "median_ms": statistics.median(ts)}
+        log(f"kernel {name}: mean {kms[name]['mean_ms']:.4f} ms, median {kms[name]['median_ms']:.4f} ms")
+
+    # executed MFMA FLOPs per selected block pair: forward 2 products, dK/dV kernel 4 (S, dP, dV, dK), dQ kernel 3
+    kernel_flops = {"fwd": 4.0 * pair_flops * nnz, "bwd_dkdv": 8.0 * pair_flops * nnz, "bwd_dq": 6.0 * pair_flops * nnz}
+    rooflines = {}
+    for name, fl in kernel_flops.items():
+        ach = fl / (kms[name]["mean_ms"] * 1e-3) * 1e-12
+        rooflines[name] = {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "ms": kms[name]["mean_ms"]}
+    dominant = max(kernel_flops, key=lambda n: kms[n]["mean_ms"])
+    roofline = dict(rooflines[dominant])
+    roofline["kernel"] = dominant
+
+    mask_bytes = mask.numel() + 4 * (2 * nnz // (1 if mask.dim() == 4 else B * H) + lists.mask_bh * (lists.nQ + lists.nK))
+    compaction = {"ms": kms["mask_compact"]["mean_ms"], "algorithmic_bytes": mask_bytes, "GB/s": mask_bytes / (kms["mask_compact"]["mean_ms"] * 1e-3) * 1e-9, "peak_GB/s": PEAK_HBM_GBS}
+    bwd_ms = kms["bwd_delta"]["mean_ms"] + kms["bwd_dkdv"]["mean_ms"] + kms["bwd_dq"]["mean_ms"]
+    detail = {
+        "fwd_ms": kms["fwd"]["mean_ms"], "fwd_TFLOP/s": fl_fwd / (kms["fwd"]["mean_ms"] * 1e-3) * 1e-12,
+        "bwd_ms": bwd_ms, "bwd_TFLOP/s": fl_bwd / (bwd_ms * 1e-3) * 1e-12,
+        "fwd+bwd_kernels_TFLOP/s": (fl_fwd + fl_bwd) / ((bwd_ms + kms["fwd"]["mean_ms"]) * 1e-3) * 1e-12,
+        "frac_of_bf16_peak": value / PEAK_BF16_TFLOPS,
+        "kernels_ms": {n: kms[n]["mean_ms"] for n in kms},
+        "rooflines": rooflines,
+        "mask_compaction": compaction,
+    }
+
+    cpu = None if args.no_cpu else cpu_baseline()
+    out = {
+        "metric": "fwd+bwd effective TFLOP/s (selected-block FLOPs), mask compaction + forward + backward",
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": w["desc"], "nnz_block_pairs": nnz, "fwd_TFLOP": fl_fwd * 1e-12, "bwd_TFLOP": fl_bwd * 1e-12},
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "detail": detail,
+    }
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()
