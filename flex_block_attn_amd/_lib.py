@@ -6,7 +6,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "csrc", "libfba_gfx950.so")
+# FBA_LIBRARY points the loader at another build of the same ABI (an instrumented or experimental one)
+LIB_PATH = os.environ.get("FBA_LIBRARY") or os.path.join(_HERE, "csrc", "libfba_gfx950.so")
 
 FBA_OK = 0
 FBA_ERR_INVALID = 1

@@ -17,6 +17,12 @@ LIB_NAME = "libfba_gfx950.so"
 LIB_PATH = os.path.join(CSRC, LIB_NAME)
 SOURCES = ["fba_api.hip", "fba_mask_compact.hip", "fba_fwd.hip", "fba_bwd.hip"]
 
+# Per-file extras.  --amdgpu-mfma-vgpr-form keeps MFMA accumulators in ordinary VGPRs, so the softmax arithmetic on
+# them needs no accumulator-register copies; it pays off where the whole working set fits 256 registers.
+EXTRA_FLAGS = {
+    "fba_fwd.hip": ["-mllvm", "--amdgpu-mfma-vgpr-form"],
+}
+
 # -packed-fp32-ops is switched off: hipcc otherwise fuses pairs of fp32 operations into packed instructions.
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
@@ -39,7 +45,7 @@ def _hipcc():
 
 def _compile_one(src, verbose):
     obj = os.path.join(CSRC, src.replace(".hip", ".o"))
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
     if verbose:
         cmd += ["-Rpass-analysis=kernel-resource-usage"]
     r = subprocess.run(cmd, capture_output=True, text=True)

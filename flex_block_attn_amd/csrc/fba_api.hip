@@ -67,7 +67,7 @@ const char* fba_last_error(void) { return g_err; }
 int32_t fba_set_option(const char* name, int32_t value) {
   if (name == nullptr) return fail(FBA_ERR_INVALID, "option name is null");
   if (std::strcmp(name, "fwd_qb") == 0) {
-    if (value < 0 || value > 3) return fail(FBA_ERR_INVALID, "fwd_qb must be 0..3, got %d", value);
+    if (value < 0 || value > 2) return fail(FBA_ERR_INVALID, "fwd_qb must be 0..2, got %d", value);
     g_fwd_qb.store(value);
     return FBA_OK;
   }
@@ -92,17 +92,13 @@ int32_t fba_fwd(const void* q, const void* k, const void* v, void* o, float* lse
   if (!lse || !q_cnt || !q_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
   if (q_block % 128 != 0)
     return fail(FBA_ERR_UNSUPPORTED, "forward: q_block (%d) must be a multiple of 128 in this build", q_block);
-  int qb = g_fwd_qb.load();
-  if (qb == 0) qb = 1;
-  if (q_block % (128 * qb) != 0) qb = 1;
-
   fba::FwdParams p{};
   p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.o = (__bf16*)o; p.lse = lse;
   p.q_cnt = q_cnt; p.q_idx = q_idx; p.mask_bh = mask_bh;
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Sq = Sq; p.Skv = Skv; p.nQ = Sq / q_block; p.nK = Skv / k_block;
   p.q_block = q_block; p.k_block = k_block;
   p.scale_log2e = 1.4426950408889634f / 11.313708498984761f;
-  hipError_t e = fba::launch_fwd(p, qb, (hipStream_t)hip_stream);
+  hipError_t e = fba::launch_fwd(p, (hipStream_t)hip_stream);
   return e == hipSuccess ? FBA_OK : hip_fail(e, "forward launch");
 }
 

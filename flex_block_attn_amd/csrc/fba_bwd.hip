@@ -84,6 +84,10 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dq_kernel
     vc.store(smem + kTileBytes, wr_off);
   }
   __syncthreads();
+  // all loads so far must have landed: inside the loop the vector-memory counter is for the slab prefetch only
+  wait_vmem_all();
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) { pin(qreg[ks]); pin(doreg[ks]); }
 
   for (int step = 0; step < nsteps; ++step) {
     const char* ks_lds = smem + (step & 1) * 2 * kTileBytes;
@@ -234,6 +238,10 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
     stash(smem);
   }
   __syncthreads();
+  // all loads so far must have landed: inside the loop the vector-memory counter is for the slab prefetch only
+  wait_vmem_all();
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) { pin(kreg[ks]); pin(vreg[ks]); }
 
   for (int step = 0; step < nsteps; ++step) {
     const char* q_lds = smem + (step & 1) * kStageBytes;

@@ -94,6 +94,13 @@ FBA_DEVICE float sum_halves(float x) {
   return p.lo + p.hi;
 }
 
+// Wait until no vector-memory load is outstanding (vmcnt = 0; expcnt and lgkmcnt fields left at their maxima).
+FBA_DEVICE void wait_vmem_all() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+// Keep a loaded value where it is: the compiler may not sink its load below this point.
+template <typename T>
+FBA_DEVICE void pin(T& v) { asm volatile("" : "+v"(v)); }
+
 FBA_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // Work-group id -> logical work item, so that each XCD (work-groups are dealt to the 8 XCDs round-robin) owns one
@@ -111,12 +118,35 @@ struct TileCopy {
 #pragma unroll
     for (int i = 0; i < kIters; ++i) reg[i] = *reinterpret_cast<const u32x4*>(p + i * 16 * kRowBytes);
   }
+  // same, from a wave-uniform byte base plus the per-thread offset (tid >> 4) * 256 + (tid & 15) * 16
+  FBA_DEVICE void load(const char* __restrict__ base, uint32_t thread_off) {
+#pragma unroll
+    for (int i = 0; i < kIters; ++i) reg[i] = *reinterpret_cast<const u32x4*>(base + thread_off + i * 16 * kRowBytes);
+  }
   // wr_off = tile_off(tid >> 4, tid & 15), precomputed by the caller
   FBA_DEVICE void store(char* tile, int wr_off) const {
 #pragma unroll
     for (int i = 0; i < kIters; ++i) *reinterpret_cast<u32x4*>(tile + wr_off + i * 16 * kRowBytes) = reg[i];
   }
 };
+
+// Address of a __shared__ object inside the work-group's LDS allocation.
+FBA_DEVICE uint32_t lds_addr(const void* p) { return (uint32_t)(uintptr_t)(FBA_LDS const char*)p; }
+
+// Direct global -> LDS copy, 16 bytes per lane: lane l's bytes land at lds_base + 16 l; it fetches them from
+// gbase + lane_off.  lds_base and gbase must be wave-uniform.  Completion is tracked by the vector-memory counter only;
+// the compiler is not told that LDS changes, so the caller orders the copy against LDS reads with wait_vmem<N>() and a
+// barrier.  (M0 carries the LDS address; one wait state separates its write from the load.)
+FBA_DEVICE void dma16(uint32_t lds_base, const char* gbase, uint32_t lane_off) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_base), "v"(lane_off), "s"(gbase)
+               : "memory", "m0");
+}
+
+// Wait until at most N vector-memory loads are outstanding (N < 16).
+template <int N>
+FBA_DEVICE void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70 | N); }
 
 // Per-lane LDS offsets for row-major A/B operand fetches of a 32-row slab: rd[ks] addresses row (lane % 32),
 // chunk 2*ks + lane/32.  Add 32*kRowBytes per further slab (rows stay congruent mod 16, so swz is unchanged).

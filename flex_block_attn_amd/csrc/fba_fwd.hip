@@ -1,29 +1,112 @@
 // Forward kernel: block-sparse softmax attention for gfx950, head_dim 128, bf16 in / fp32 accumulate.
 //
-// One work-group of 4 waves owns 128*QB consecutive query rows of one (batch, head); wave w owns rows
-// [32*QB*w, 32*QB*(w+1)).  The work-group walks the active-key-block list of its query block and streams every
-// selected key block through LDS as 64-key slabs of K and V (two stages, one barrier per slab).
+// One work-group of 4 waves owns 128 consecutive query rows of one (batch, head); wave w owns rows [32w, 32w+32).
+// The work-group walks the active-key-block list of its query block and streams every selected key block through
+// LDS as 64-key slabs of K and V (two buffers each).
 //
-// Per slab and wave, in "transposed" form so that softmax statistics are per-lane scalars:
+// Everything is kept "transposed" so that softmax statistics are per-lane scalars (lane = query row):
 //   S^T[key, q]  = K[key, :] . Q[q, :]            A = K slab rows from LDS (128-bit fetches), B = Q in registers
-//   P^T          = exp2(c * S^T - c * m[q])        fp32, c = log2(e) / sqrt(128); running max m and sum l per lane
+//   P^T          = exp2(c * S^T - c * m[q])        fp32, c = log2(e) / sqrt(128); running reference m and sum l per lane
 //   O^T[d, q]   += V^T[d, key] . P^T[key, q]       A = V slab through transposing LDS fetches, B = P^T packed to bf16
 // The reference computes the same quantities per selected tile (flex_block_attn_h100.cu:245-290, online softmax
 // :199-221, final O / l at :292); here LSE is stored as the natural-log value m/sqrt(128) + ln(l).
+//
+// Software pipeline.  The unit of work is a 32-key slab t.  While the VALU turns S_t into P_t, the matrix pipe computes
+// S_{t+1} and adds P_{t-1} V_{t-1} into O; the three are independent, so one wave keeps both pipes busy.
+// K and V slabs travel global -> LDS directly (no registers) into two rings of four 8 KiB buffers: after step t the
+// buffers of K_{t+1} and V_{t-1} are dead and receive K_{t+5} and V_{t+3}, i.e. every slab is requested four steps
+// before its first use.  One barrier per step orders all LDS traffic; before it each wave waits until its own copies
+// of the slabs needed next have landed (all but the two youngest batches of four).
+#include <type_traits>
+
 #include "fba_common.h"
 #include "fba_kernels.h"
 
 namespace fba {
 
-template <int QB>
-__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void fwd_kernel(const FwdParams p) {
-  extern __shared__ __attribute__((aligned(16))) char smem[];
-  constexpr int TQ = 128 * QB;
-  constexpr int kSlab = 64;
-  constexpr int kTileBytes = kSlab * kRowBytes;  // 16 KiB
-  // smem: [stage][K | V]
+namespace {
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+constexpr int kSlab = 32;                      // keys per LDS slab
+constexpr int kSlabBytes = kSlab * kRowBytes;  // 8 KiB
+constexpr int kRing = 4;                       // slabs per ring
+constexpr float kLazy = 8.f;                   // log2 headroom before the softmax reference is raised
+
+template <int N>
+using IC = std::integral_constant<int, N>;
+
+struct FwdState {
+  bf16x8 qreg[8];
+  f32x16 acc_o[4];
+  float m_run, l_run;
+  RowMajorOffsets rm;
+  TransposedOffsets tr;
+  float c;
+};
+
+// S^T for 32 keys: 8 MFMAs.  k_half points at the first of the 32 key rows inside a swizzled slab.
+FBA_DEVICE f32x16 qk_half(const FwdState& st, const char* k_half) {
+  f32x16 s;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) s = mfma32(lds_read_b128(k_half, st.rm.rd[ks]), st.qreg[ks], s);
+  return s;
+}
+
+// O^T += V^T P^T for 32 keys: 8 MFMAs.  Consecutive MFMAs go to different accumulators.
+FBA_DEVICE void pv_half(FwdState& st, const char* v_half, const bf16x8 (&pk)[2]) {
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+      const int roff = 16 * j * kRowBytes;
+      const bf16x8 a = cat(lds_read_tr(v_half, st.tr.rd[mb][0] + roff), lds_read_tr(v_half, st.tr.rd[mb][1] + roff));
+      st.acc_o[mb] = mfma32(a, pk[j], st.acc_o[mb]);
+    }
+}
+
+// Raise the softmax reference if some row of the wave would otherwise see exponents above kLazy.  Until then
+// P = exp2(c (S - m)) may exceed 1, which fp32 sums and bf16 P both carry.
+FBA_DEVICE void softmax_reference(FwdState& st, const f32x16& s) {
+  float mx = s[0];
+#pragma unroll
+  for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[r]);
+  mx = max_halves(mx);
+  if (__builtin_amdgcn_ballot_w64((mx - st.m_run) * st.c > kLazy) != 0) {
+    const float m_new = fmaxf(st.m_run, mx);
+    const float alpha = fast_exp2((st.m_run - m_new) * st.c);
+    st.m_run = m_new;
+    st.l_run *= alpha;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) st.acc_o[mb][r] *= alpha;
+  }
+}
+
+// P^T = exp2(c S^T - c m), row sums into l, packed to bf16 as the B operand of the two 16-key MFMA steps.
+FBA_DEVICE void softmax_exp(FwdState& st, f32x16& s, bf16x8 (&pk)[2]) {
+  const float mc = st.m_run * st.c;
+  float rs = 0.f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    s[r] = fast_exp2(__builtin_fmaf(s[r], st.c, -mc));
+    rs += s[r];
+  }
+  st.l_run += rs;
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+    pk[j] = pack8(s[8 * j + 0], s[8 * j + 1], s[8 * j + 2], s[8 * j + 3], s[8 * j + 4], s[8 * j + 5], s[8 * j + 6], s[8 * j + 7]);
+}
+
+}  // namespace
+
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_per_eu(2, 2))) void fwd_kernel(const FwdParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];  // K ring [4][8 KiB] | V ring [4][8 KiB]
+  constexpr int TQ = 128;
+
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int item = xcd_remap(blockIdx.x, p.items_per_xcd);
   if (item >= p.num_items) return;
   const int tiles_per_head = p.Sq / TQ;
@@ -32,9 +115,10 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void fwd_kerne
   const int b = bh / p.Hq, hq = bh - b * p.Hq;
   const int hkv = hq / (p.Hq / p.Hkv);
 
-  const __bf16* qp = p.q + ((int64_t)bh * p.Sq + (int64_t)qt * TQ + wave * 32 * QB) * kHeadDim;
-  const __bf16* kp = p.k + ((int64_t)(b * p.Hkv + hkv) * p.Skv) * kHeadDim;
-  const __bf16* vp = p.v + ((int64_t)(b * p.Hkv + hkv) * p.Skv) * kHeadDim;
+  const int64_t qrow0 = (int64_t)bh * p.Sq + (int64_t)qt * TQ + wave * 32;
+  const __bf16* qp = p.q + qrow0 * kHeadDim;
+  const char* kp = reinterpret_cast<const char*>(p.k + ((int64_t)(b * p.Hkv + hkv) * p.Skv) * kHeadDim);
+  const char* vp = reinterpret_cast<const char*>(p.v + ((int64_t)(b * p.Hkv + hkv) * p.Skv) * kHeadDim);
 
   const int qblk = (qt * TQ) / p.q_block;
   const int64_t mrow = (p.mask_bh == 1 ? 0 : (int64_t)bh) * p.nQ + qblk;
@@ -43,167 +127,132 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void fwd_kerne
   const int nsub = p.k_block / kSlab;
   const int nsteps = cnt * nsub;
 
-  // Q as the B operand: lane holds row (32 n + l32), d = 16 ks + 8 h .. +7
-  bf16x8 qreg[QB][8];
+  FwdState st;
+  // Q as the B operand: lane holds row l32, d = 16 ks + 8 h .. +7
 #pragma unroll
-  for (int n = 0; n < QB; ++n)
+  for (int ks = 0; ks < 8; ++ks) st.qreg[ks] = *reinterpret_cast<const bf16x8*>(qp + (int64_t)l32 * kHeadDim + 16 * ks + 8 * h);
+  st.rm.init(lane);
+  st.tr.init(lane);
+  st.c = p.scale_log2e;
+  st.m_run = -INFINITY;
+  st.l_run = 0.f;
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks)
-      qreg[n][ks] = *reinterpret_cast<const bf16x8*>(qp + (int64_t)(32 * n + l32) * kHeadDim + 16 * ks + 8 * h);
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) st.acc_o[mb][r] = 0.f;
 
-  RowMajorOffsets rm;
-  rm.init(lane);
-  TransposedOffsets tr;
-  tr.init(lane);
-  const int wr_off = tile_off(tid >> 4, tid & 15);
-
-  f32x16 acc_o[QB][4];
-  float m_run[QB], l_run[QB];
+  // Slab copies.  A wave-level copy fills 1 KiB = 4 rows of a slab; wave w owns rows 8w .. 8w+7 (two copies).  Lane l
+  // lands in row 4g + l/16, chunk slot l%16, so it must fetch chunk (l%16) ^ swz(row) of that row.
+  uint32_t dma_off[2];
 #pragma unroll
-  for (int n = 0; n < QB; ++n) {
-    m_run[n] = -INFINITY;
-    l_run[n] = 0.f;
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc_o[n][mb][r] = 0.f;
+  for (int g = 0; g < 2; ++g) {
+    const int row = 8 * wave + 4 * g + (lane >> 4);
+    dma_off[g] = (uint32_t)(row * kRowBytes + (((lane & 15) ^ swz(row)) << 4));
   }
-  const float c = p.scale_log2e;
+  char* const k_lds = smem;
+  char* const v_lds = smem + kRing * kSlabBytes;
+  const uint32_t k_dst = lds_addr(k_lds) + wave * 8 * kRowBytes;
+  const uint32_t v_dst = lds_addr(v_lds) + wave * 8 * kRowBytes;
 
-  TileCopy<kSlab> kc, vc;
-  int e_next = 0, s_next = 0;  // list entry / slab of the next tile to fetch
-  auto fetch = [&]() {
-    const int64_t row0 = (int64_t)idx[e_next] * p.k_block + s_next * kSlab;
-    kc.load(kp + row0 * kHeadDim, tid);
-    vc.load(vp + row0 * kHeadDim, tid);
-    if (++s_next == nsub) { s_next = 0; ++e_next; }
+  // K and V each walk the list with their own cursor (K runs two slabs ahead of V); the list entry of the following
+  // key block is read one block ahead, so that the scalar load is off the critical path.
+  struct Cursor {
+    int e, s, blk;
+  };
+  auto advance = [&](Cursor& cu) -> int64_t {
+    const int64_t byte0 = ((int64_t)cu.blk * p.k_block + cu.s * kSlab) * kRowBytes;
+    if (++cu.s == nsub) {
+      cu.s = 0;
+      ++cu.e;
+      cu.blk = cu.e < cnt ? idx[cu.e] : 0;
+    }
+    return byte0;
+  };
+  const int blk0 = cnt > 0 ? idx[0] : 0;
+  Cursor kcur{0, 0, blk0}, vcur{0, 0, blk0};
+  auto copy_k = [&](int ring) {  // next K slab -> ring buffer
+    const char* src = kp + advance(kcur);
+    dma16(k_dst + ring * kSlabBytes, src, dma_off[0]);
+    dma16(k_dst + ring * kSlabBytes + 4 * kRowBytes, src, dma_off[1]);
+  };
+  auto copy_v = [&](int ring) {
+    const char* src = vp + advance(vcur);
+    dma16(v_dst + ring * kSlabBytes, src, dma_off[0]);
+    dma16(v_dst + ring * kSlabBytes + 4 * kRowBytes, src, dma_off[1]);
   };
 
   if (nsteps > 0) {
-    fetch();
-    kc.store(smem, wr_off);
-    vc.store(smem + kTileBytes, wr_off);
-  }
-  __syncthreads();
-
-  for (int step = 0; step < nsteps; ++step) {
-    const char* ks_lds = smem + (step & 1) * 2 * kTileBytes;
-    const char* vs_lds = ks_lds + kTileBytes;
-    char* nxt = smem + ((step + 1) & 1) * 2 * kTileBytes;
-    const bool more = step + 1 < nsteps;
-    if (more) fetch();
-
-    // S^T = K Q^T
-    f32x16 s[QB][2];
+    // prologue: K_0..K_3 and V_0..V_2 requested, S_0 computed, then K_4 into the buffer of K_0
 #pragma unroll
-    for (int n = 0; n < QB; ++n)
+    for (int j = 0; j < 4; ++j)
+      if (j < nsteps) copy_k(j);
 #pragma unroll
-      for (int m2 = 0; m2 < 2; ++m2)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) s[n][m2][r] = 0.f;
-#pragma unroll
-    for (int m2 = 0; m2 < 2; ++m2)
-#pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        const bf16x8 a = lds_read_b128(ks_lds, rm.rd[ks] + m2 * 32 * kRowBytes);
-#pragma unroll
-        for (int n = 0; n < QB; ++n) s[n][m2] = mfma32(a, qreg[n][ks], s[n][m2]);
-      }
-
-    // online softmax, per lane (= per query row; the two half-waves hold disjoint keys of the same row)
-    bf16x8 pk[QB][2][2];
-#pragma unroll
-    for (int n = 0; n < QB; ++n) {
-      float mx = m_run[n];
-#pragma unroll
-      for (int m2 = 0; m2 < 2; ++m2)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[n][m2][r]);
-      mx = max_halves(mx);
-      const float alpha = fast_exp2((m_run[n] - mx) * c);
-      m_run[n] = mx;
-      const float mc = mx * c;
-      float rs = 0.f;
-#pragma unroll
-      for (int m2 = 0; m2 < 2; ++m2)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const float pv = fast_exp2(__builtin_fmaf(s[n][m2][r], c, -mc));
-          s[n][m2][r] = pv;
-          rs += pv;
-        }
-      l_run[n] = l_run[n] * alpha + rs;
-#pragma unroll
-      for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc_o[n][mb][r] *= alpha;
-#pragma unroll
-      for (int m2 = 0; m2 < 2; ++m2)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-          pk[n][m2][j] = pack8(s[n][m2][8 * j + 0], s[n][m2][8 * j + 1], s[n][m2][8 * j + 2], s[n][m2][8 * j + 3],
-                               s[n][m2][8 * j + 4], s[n][m2][8 * j + 5], s[n][m2][8 * j + 6], s[n][m2][8 * j + 7]);
-    }
-
-    // O^T += V^T P^T
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-      for (int m2 = 0; m2 < 2; ++m2)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-          const int roff = (32 * m2 + 16 * j) * kRowBytes;
-          const bf16x8 a = cat(lds_read_tr(vs_lds, tr.rd[mb][0] + roff), lds_read_tr(vs_lds, tr.rd[mb][1] + roff));
-#pragma unroll
-          for (int n = 0; n < QB; ++n) acc_o[n][mb] = mfma32(a, pk[n][m2][j], acc_o[n][mb]);
-        }
-
-    if (more) {
-      kc.store(nxt, wr_off);
-      vc.store(nxt + kTileBytes, wr_off);
-    }
+    for (int j = 0; j < 3; ++j)
+      if (j < nsteps) copy_v(j);
+    wait_vmem<0>();
     __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) pin(st.qreg[ks]);
+    f32x16 s_cur = qk_half(st, k_lds);
+    pin(s_cur);
+    __syncthreads();
+    if (4 < nsteps) copy_k(0);
+
+    bf16x8 p_prev[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int t = 0; t < 8; ++t) p_prev[j][t] = (__bf16)0.f;
+
+    // step t (t % 4 == R): softmax(S_t) | S_{t+1} = K_{t+1} Q^T | O += P_{t-1} V_{t-1}
+    auto step = [&](auto ring_c, int t) {
+      constexpr int R = decltype(ring_c)::value;
+      softmax_reference(st, s_cur);
+      const f32x16 s_nxt = qk_half(st, k_lds + ((R + 1) & 3) * kSlabBytes);  // past the last slab: stale data, unused
+      // P of "slab -1" is zero; any finite V will do for it
+      pv_half(st, t == 0 ? v_lds : v_lds + ((R + 3) & 3) * kSlabBytes, p_prev);
+      softmax_exp(st, s_cur, p_prev);  // p_prev := P_t
+      s_cur = s_nxt;
+      // K_{t+2} and V_t must have landed; the copies requested after steps t-2 and t-1 (4 each) may still fly
+      if (t + 5 < nsteps) wait_vmem<8>(); else wait_vmem<0>();
+      __syncthreads();
+      if (t + 5 < nsteps) copy_k((R + 1) & 3);
+      if (t + 3 < nsteps) copy_v((R + 3) & 3);
+    };
+    for (int t = 0; t < nsteps; t += 4) {
+      step(IC<0>{}, t);
+      step(IC<1>{}, t + 1);
+      if (t + 2 >= nsteps) break;  // nsteps is even
+      step(IC<2>{}, t + 2);
+      step(IC<3>{}, t + 3);
+    }
+    // O += P_{n-1} V_{n-1}
+    pv_half(st, v_lds + ((nsteps - 1) & 3) * kSlabBytes, p_prev);
   }
 
   // epilogue: O = O^T / l, LSE = ln2 * (c m + log2 l)
-  __bf16* op = p.o + ((int64_t)bh * p.Sq + (int64_t)qt * TQ + wave * 32 * QB) * kHeadDim;
-  float* lp = p.lse + (int64_t)bh * p.Sq + (int64_t)qt * TQ + wave * 32 * QB;
+  __bf16* orow = p.o + (qrow0 + l32) * kHeadDim;
+  const float l = sum_halves(st.l_run);
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  if (h == 0) p.lse[qrow0 + l32] = l > 0.f ? (st.m_run * st.c + __builtin_log2f(l)) * 0.6931471805599453f : -INFINITY;
 #pragma unroll
-  for (int n = 0; n < QB; ++n) {
-    const float l = sum_halves(l_run[n]);
-    const float inv = l > 0.f ? 1.f / l : 0.f;
-    if (h == 0) lp[32 * n + l32] = l > 0.f ? (m_run[n] * c + __builtin_log2f(l)) * 0.6931471805599453f : -INFINITY;
-    __bf16* orow = op + (int64_t)(32 * n + l32) * kHeadDim;
+  for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
-    for (int mb = 0; mb < 4; ++mb)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const bf16x4 ov = pack4(acc_o[n][mb][4 * g + 0] * inv, acc_o[n][mb][4 * g + 1] * inv,
-                                acc_o[n][mb][4 * g + 2] * inv, acc_o[n][mb][4 * g + 3] * inv);
-        *reinterpret_cast<bf16x4*>(orow + 32 * mb + 8 * g + 4 * h) = ov;
-      }
-  }
+    for (int g = 0; g < 4; ++g) {
+      const bf16x4 ov = pack4(st.acc_o[mb][4 * g + 0] * inv, st.acc_o[mb][4 * g + 1] * inv, st.acc_o[mb][4 * g + 2] * inv,
+                              st.acc_o[mb][4 * g + 3] * inv);
+      *reinterpret_cast<bf16x4*>(orow + 32 * mb + 8 * g + 4 * h) = ov;
+    }
 }
 
-template <int QB>
-static hipError_t launch(const FwdParams& p, hipStream_t stream) {
-  constexpr int kSmem = 2 * 2 * 64 * kRowBytes;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel<QB>), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
-  if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(fwd_kernel<QB>, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
-  return hipGetLastError();
-}
-
-hipError_t launch_fwd(FwdParams p, int qb, hipStream_t stream) {
-  const int tq = 128 * qb;
-  p.num_items = p.B * p.Hq * (p.Sq / tq);
+hipError_t launch_fwd(FwdParams p, hipStream_t stream) {
+  constexpr int kSmem = 2 * kRing * kSlabBytes;
+  p.num_items = p.B * p.Hq * (p.Sq / 128);
   p.items_per_xcd = (p.num_items + kNumXcd - 1) / kNumXcd;
-  switch (qb) {
-    case 1: return launch<1>(p, stream);
-    case 2: return launch<2>(p, stream);
-    case 3: return launch<3>(p, stream);
-    default: return hipErrorInvalidValue;
-  }
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(fwd_kernel, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
+  return hipGetLastError();
 }
 
 }  // namespace fba
