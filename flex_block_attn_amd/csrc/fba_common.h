@@ -30,6 +30,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 #define FBA_LDS __attribute__((address_space(3)))
+#define FBA_CONST __attribute__((address_space(4)))
 #define FBA_DEVICE __device__ __forceinline__
 
 constexpr int kHeadDim = 128;
@@ -130,18 +131,23 @@ struct TileCopy {
   }
 };
 
+// Read-only view of a block-index list in global memory.  Loads through the constant address space stay scalar loads
+// (s_load_dword) wherever they sit, also behind inline asm and barriers.
+typedef const FBA_CONST int32_t* ConstIdx;
+FBA_DEVICE ConstIdx const_idx(const int32_t* p) { return (ConstIdx)(uintptr_t)p; }
+
 // Address of a __shared__ object inside the work-group's LDS allocation.
 FBA_DEVICE uint32_t lds_addr(const void* p) { return (uint32_t)(uintptr_t)(FBA_LDS const char*)p; }
 
 // Direct global -> LDS copy, 16 bytes per lane: lane l's bytes land at lds_base + 16 l; it fetches them from
 // gbase + lane_off.  lds_base and gbase must be wave-uniform.  Completion is tracked by the vector-memory counter only;
-// the compiler is not told that LDS changes, so the caller orders the copy against LDS reads with wait_vmem<N>() and a
-// barrier.  (M0 carries the LDS address; one wait state separates its write from the load.)
+// the compiler is not told that LDS changes (no memory clobber either: that would turn the scalar loads of the block
+// lists into vector loads), so the caller orders the copy against LDS reads with wait_vmem<N>() and a barrier.  (M0 carries the LDS address; one wait state separates its write from the load.)
 FBA_DEVICE void dma16(uint32_t lds_base, const char* gbase, uint32_t lane_off) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
                : "s"(lds_base), "v"(lane_off), "s"(gbase)
-               : "memory", "m0");
+               : "m0");
 }
 
 // Wait until at most N vector-memory loads are outstanding (N < 16).

@@ -37,7 +37,9 @@ using IC = std::integral_constant<int, N>;
 struct FwdState {
   bf16x8 qreg[8];
   f32x16 acc_o[4];
-  float m_run, l_run;
+  f32x16 acc_l;  // every element of a lane: sum over keys of bf16(P) for the lane's query row
+  bf16x8 ones;
+  float m_run;
   RowMajorOffsets rm;
   TransposedOffsets tr;
   float c;
@@ -53,16 +55,20 @@ FBA_DEVICE f32x16 qk_half(const FwdState& st, const char* k_half) {
   return s;
 }
 
-// O^T += V^T P^T for 32 keys: 8 MFMAs.  Consecutive MFMAs go to different accumulators.
+// O^T += V^T P^T for 32 keys: 8 MFMAs, plus 2 with an all-ones A operand that accumulate the softmax denominator
+// (sum over keys of the same bf16 P that weighs V) without spending VALU additions on it.  Consecutive MFMAs go to
+// different accumulators.
 FBA_DEVICE void pv_half(FwdState& st, const char* v_half, const bf16x8 (&pk)[2]) {
 #pragma unroll
-  for (int j = 0; j < 2; ++j)
+  for (int j = 0; j < 2; ++j) {
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
       const int roff = 16 * j * kRowBytes;
       const bf16x8 a = cat(lds_read_tr(v_half, st.tr.rd[mb][0] + roff), lds_read_tr(v_half, st.tr.rd[mb][1] + roff));
       st.acc_o[mb] = mfma32(a, pk[j], st.acc_o[mb]);
     }
+    st.acc_l = mfma32(st.ones, pk[j], st.acc_l);
+  }
 }
 
 // Raise the softmax reference if some row of the wave would otherwise see exponents above kLazy.  Until then
@@ -76,7 +82,8 @@ FBA_DEVICE void softmax_reference(FwdState& st, const f32x16& s) {
     const float m_new = fmaxf(st.m_run, mx);
     const float alpha = fast_exp2((st.m_run - m_new) * st.c);
     st.m_run = m_new;
-    st.l_run *= alpha;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) st.acc_l[r] *= alpha;
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
@@ -84,16 +91,11 @@ FBA_DEVICE void softmax_reference(FwdState& st, const f32x16& s) {
   }
 }
 
-// P^T = exp2(c S^T - c m), row sums into l, packed to bf16 as the B operand of the two 16-key MFMA steps.
+// P^T = exp2(c S^T - c m), packed to bf16 as the B operand of the two 16-key MFMA steps.
 FBA_DEVICE void softmax_exp(FwdState& st, f32x16& s, bf16x8 (&pk)[2]) {
   const float mc = st.m_run * st.c;
-  float rs = 0.f;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    s[r] = fast_exp2(__builtin_fmaf(s[r], st.c, -mc));
-    rs += s[r];
-  }
-  st.l_run += rs;
+  for (int r = 0; r < 16; ++r) s[r] = fast_exp2(__builtin_fmaf(s[r], st.c, -mc));
 #pragma unroll
   for (int j = 0; j < 2; ++j)
     pk[j] = pack8(s[8 * j + 0], s[8 * j + 1], s[8 * j + 2], s[8 * j + 3], s[8 * j + 4], s[8 * j + 5], s[8 * j + 6], s[8 * j + 7]);
@@ -123,7 +125,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   const int qblk = (qt * TQ) / p.q_block;
   const int64_t mrow = (p.mask_bh == 1 ? 0 : (int64_t)bh) * p.nQ + qblk;
   const int cnt = p.q_cnt[mrow];
-  const int32_t* __restrict__ idx = p.q_idx + mrow * p.nK;
+  const ConstIdx idx = const_idx(p.q_idx + mrow * p.nK);
   const int nsub = p.k_block / kSlab;
   const int nsteps = cnt * nsub;
 
@@ -135,7 +137,10 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   st.tr.init(lane);
   st.c = p.scale_log2e;
   st.m_run = -INFINITY;
-  st.l_run = 0.f;
+#pragma unroll
+  for (int t = 0; t < 8; ++t) st.ones[t] = (__bf16)1.f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) st.acc_l[r] = 0.f;
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
@@ -154,41 +159,41 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   const uint32_t k_dst = lds_addr(k_lds) + wave * 8 * kRowBytes;
   const uint32_t v_dst = lds_addr(v_lds) + wave * 8 * kRowBytes;
 
-  // K and V each walk the list with their own cursor (K runs two slabs ahead of V); the list entry of the following
-  // key block is read one block ahead, so that the scalar load is off the critical path.
-  struct Cursor {
-    int e, s, blk;
-  };
-  auto advance = [&](Cursor& cu) -> int64_t {
-    const int64_t byte0 = ((int64_t)cu.blk * p.k_block + cu.s * kSlab) * kRowBytes;
-    if (++cu.s == nsub) {
-      cu.s = 0;
-      ++cu.e;
-      cu.blk = cu.e < cnt ? idx[cu.e] : 0;
+  // Slab source offsets, in list order.  The list entry of the following key block is read one block ahead, so that
+  // the scalar load is off the critical path.  V requests trail K requests by two slabs and reuse their offsets.
+  const int64_t block_bytes = (int64_t)p.k_block * kRowBytes;
+  int e_next = 1, rem = nsub;
+  int64_t src_off = cnt > 0 ? idx[0] * block_bytes : 0;
+  int blk_next = cnt > 1 ? idx[1] : 0;
+  auto next_off = [&]() -> int64_t {
+    const int64_t off = src_off;
+    if (--rem == 0) {
+      rem = nsub;
+      src_off = blk_next * block_bytes;
+      ++e_next;
+      blk_next = e_next < cnt ? idx[e_next] : 0;
+    } else {
+      src_off += kSlabBytes;
     }
-    return byte0;
+    return off;
   };
-  const int blk0 = cnt > 0 ? idx[0] : 0;
-  Cursor kcur{0, 0, blk0}, vcur{0, 0, blk0};
-  auto copy_k = [&](int ring) {  // next K slab -> ring buffer
-    const char* src = kp + advance(kcur);
-    dma16(k_dst + ring * kSlabBytes, src, dma_off[0]);
-    dma16(k_dst + ring * kSlabBytes + 4 * kRowBytes, src, dma_off[1]);
-  };
-  auto copy_v = [&](int ring) {
-    const char* src = vp + advance(vcur);
-    dma16(v_dst + ring * kSlabBytes, src, dma_off[0]);
-    dma16(v_dst + ring * kSlabBytes + 4 * kRowBytes, src, dma_off[1]);
+  auto copy_slab = [&](uint32_t dst, const char* src) {
+    dma16(dst, src, dma_off[0]);
+    dma16(dst + 4 * kRowBytes, src, dma_off[1]);
   };
 
   if (nsteps > 0) {
     // prologue: K_0..K_3 and V_0..V_2 requested, S_0 computed, then K_4 into the buffer of K_0
+    int64_t off[5] = {0, 0, 0, 0, 0};
 #pragma unroll
     for (int j = 0; j < 4; ++j)
-      if (j < nsteps) copy_k(j);
+      if (j < nsteps) {
+        off[j] = next_off();
+        copy_slab(k_dst + j * kSlabBytes, kp + off[j]);
+      }
 #pragma unroll
     for (int j = 0; j < 3; ++j)
-      if (j < nsteps) copy_v(j);
+      if (j < nsteps) copy_slab(v_dst + j * kSlabBytes, vp + off[j]);
     wait_vmem<0>();
     __syncthreads();
 #pragma unroll
@@ -196,35 +201,46 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     f32x16 s_cur = qk_half(st, k_lds);
     pin(s_cur);
     __syncthreads();
-    if (4 < nsteps) copy_k(0);
+    if (4 < nsteps) {
+      off[4] = next_off();
+      copy_slab(k_dst, kp + off[4]);
+    }
+    int64_t hist0 = off[4], hist1 = off[3];  // offsets of the two youngest K requests
 
     bf16x8 p_prev[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int t = 0; t < 8; ++t) p_prev[j][t] = (__bf16)0.f;
 
     // step t (t % 4 == R): softmax(S_t) | S_{t+1} = K_{t+1} Q^T | O += P_{t-1} V_{t-1}
-    auto step = [&](auto ring_c, int t) {
+    auto step = [&](auto ring_c, auto first_c, int t) {
       constexpr int R = decltype(ring_c)::value;
+      constexpr bool kFirst = decltype(first_c)::value;
       softmax_reference(st, s_cur);
       const f32x16 s_nxt = qk_half(st, k_lds + ((R + 1) & 3) * kSlabBytes);  // past the last slab: stale data, unused
-      // P of "slab -1" is zero; any finite V will do for it
-      pv_half(st, t == 0 ? v_lds : v_lds + ((R + 3) & 3) * kSlabBytes, p_prev);
+      if constexpr (!kFirst) pv_half(st, v_lds + ((R + 3) & 3) * kSlabBytes, p_prev);
       softmax_exp(st, s_cur, p_prev);  // p_prev := P_t
+      // P_t is only consumed after the barrier; without the pins its arithmetic sinks there, away from the MFMAs it is
+      // meant to overlap with
+      pin(p_prev[0]);
+      pin(p_prev[1]);
       s_cur = s_nxt;
       // K_{t+2} and V_t must have landed; the copies requested after steps t-2 and t-1 (4 each) may still fly
       if (t + 5 < nsteps) wait_vmem<8>(); else wait_vmem<0>();
       __syncthreads();
-      if (t + 5 < nsteps) copy_k((R + 1) & 3);
-      if (t + 3 < nsteps) copy_v((R + 3) & 3);
+      const int64_t v_off = hist1;
+      hist1 = hist0;
+      if (t + 5 < nsteps) {
+        hist0 = next_off();
+        copy_slab(k_dst + ((R + 1) & 3) * kSlabBytes, kp + hist0);
+      }
+      if (t + 3 < nsteps) copy_slab(v_dst + ((R + 3) & 3) * kSlabBytes, vp + v_off);
     };
-    for (int t = 0; t < nsteps; t += 4) {
-      step(IC<0>{}, t);
-      step(IC<1>{}, t + 1);
-      if (t + 2 >= nsteps) break;  // nsteps is even
-      step(IC<2>{}, t + 2);
-      step(IC<3>{}, t + 3);
+    step(IC<0>{}, std::true_type{}, 0);
+    step(IC<1>{}, std::false_type{}, 1);
+    for (int t = 2; t < nsteps; t += 4) {  // nsteps is even
+      step(IC<2>{}, std::false_type{}, t);
+      step(IC<3>{}, std::false_type{}, t + 1);
+      if (t + 2 >= nsteps) break;
+      step(IC<0>{}, std::false_type{}, t + 2);
+      step(IC<1>{}, std::false_type{}, t + 3);
     }
     // O += P_{n-1} V_{n-1}
     pv_half(st, v_lds + ((nsteps - 1) & 3) * kSlabBytes, p_prev);
@@ -232,7 +248,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 
   // epilogue: O = O^T / l, LSE = ln2 * (c m + log2 l)
   __bf16* orow = p.o + (qrow0 + l32) * kHeadDim;
-  const float l = sum_halves(st.l_run);
+  const float l = st.acc_l[0];
   const float inv = l > 0.f ? 1.f / l : 0.f;
   if (h == 0) p.lse[qrow0 + l32] = l > 0.f ? (st.m_run * st.c + __builtin_log2f(l)) * 0.6931471805599453f : -INFINITY;
 #pragma unroll
