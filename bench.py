@@ -3,7 +3,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload random|full|sta|ssta] [--no-cpu]
 
-One step = mask compaction + forward + backward (delta, dK/dV, dQ) on synthetic inputs already resident in HBM.
+One step = mask compaction + forward + backward (statistics, dK/dV, dQ) on synthetic inputs already resident in HBM.
 Default workload: B=1, H=24, S=30720, head_dim 128, bf16, 384-token blocks (80x80), an independent random mask per
 (batch, head) keeping 32 of 80 key blocks per query-block row with the diagonal forced on.
 FLOPs count selected block pairs only: forward 4*Bq*Bk*D, backward 10*Bq*Bk*D per pair.
@@ -107,7 +107,6 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="random")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--fwd-qb", type=int, default=0, help="tuning: forward work-group height in units of 128 rows")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU only: every box in this build has a single MI355X (use --gpus 1)")
@@ -119,8 +118,6 @@ def main():
     from flex_block_attn_amd.interface import _ptr, _stream
 
     _lib.load()
-    if args.fwd_qb:
-        _lib.call("fba_set_option", b"fwd_qb", args.fwd_qb)
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     w = build_workload(args.workload, dev)
@@ -151,15 +148,15 @@ def main():
     lists = fba.compact_block_mask(mask)
     o, lse = fba.forward_with_lists(q, k, v, qbs, kbs, lists)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    delta = torch.empty((B, H, S), dtype=torch.float32, device=dev)
+    stats = torch.empty((2, B, H, S), dtype=torch.float32, device=dev)
     o2, lse2 = torch.empty_like(o), torch.empty_like(lse)
     common = (lists.mask_bh, B, H, H, S, S, D, qbs, kbs)
     kernels = {
         "mask_compact": lambda: _lib.call("fba_mask_compact", _ptr(mask), lists.mask_bh, lists.nQ, lists.nK, _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), _stream()),
         "fwd": lambda: _lib.call("fba_fwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o2), _ptr(lse2), _ptr(lists.q_cnt), _ptr(lists.q_idx), *common, _stream()),
-        "bwd_delta": lambda: _lib.call("fba_bwd_delta", _ptr(o), _ptr(do), _ptr(delta), B * H * S, D, _stream()),
-        "bwd_dkdv": lambda: _lib.call("fba_bwd_dkdv", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(lse), _ptr(delta), _ptr(dk), _ptr(dv), _ptr(lists.k_cnt), _ptr(lists.k_idx), *common, _stream()),
-        "bwd_dq": lambda: _lib.call("fba_bwd_dq", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(lse), _ptr(delta), _ptr(dq), _ptr(lists.q_cnt), _ptr(lists.q_idx), *common, _stream()),
+        "bwd_stats": lambda: _lib.call("fba_bwd_stats", _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), B * H * S, D, _stream()),
+        "bwd_dkdv": lambda: _lib.call("fba_bwd_dkdv", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(stats), _ptr(dk), _ptr(dv), _ptr(lists.k_cnt), _ptr(lists.k_idx), *common, _stream()),
+        "bwd_dq": lambda: _lib.call("fba_bwd_dq", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(stats), _ptr(dq), _ptr(lists.q_cnt), _ptr(lists.q_idx), *common, _stream()),
     }
     iters = max(5, args.steps)
     kms = {}
@@ -180,7 +177,7 @@ def main():
 
     mask_bytes = mask.numel() + 4 * (2 * nnz // (1 if mask.dim() == 4 else B * H) + lists.mask_bh * (lists.nQ + lists.nK))
     compaction = {"ms": kms["mask_compact"]["mean_ms"], "algorithmic_bytes": mask_bytes, "GB/s": mask_bytes / (kms["mask_compact"]["mean_ms"] * 1e-3) * 1e-9, "peak_GB/s": PEAK_HBM_GBS}
-    bwd_ms = kms["bwd_delta"]["mean_ms"] + kms["bwd_dkdv"]["mean_ms"] + kms["bwd_dq"]["mean_ms"]
+    bwd_ms = kms["bwd_stats"]["mean_ms"] + kms["bwd_dkdv"]["mean_ms"] + kms["bwd_dq"]["mean_ms"]
     detail = {
         "fwd_ms": kms["fwd"]["mean_ms"], "fwd_TFLOP/s": fl_fwd / (kms["fwd"]["mean_ms"] * 1e-3) * 1e-12,
         "bwd_ms": bwd_ms, "bwd_TFLOP/s": fl_bwd / (bwd_ms * 1e-3) * 1e-12,

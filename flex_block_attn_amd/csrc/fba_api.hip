@@ -1,5 +1,4 @@
 // C ABI entry points: argument validation, variant selection, launches.  See include/fba.h for the contract.
-#include <atomic>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -10,7 +9,6 @@
 namespace {
 
 thread_local char g_err[512] = "";
-std::atomic<int> g_fwd_qb{0};
 
 int fail(int code, const char* fmt, ...) {
   va_list ap;
@@ -66,11 +64,6 @@ const char* fba_last_error(void) { return g_err; }
 
 int32_t fba_set_option(const char* name, int32_t value) {
   if (name == nullptr) return fail(FBA_ERR_INVALID, "option name is null");
-  if (std::strcmp(name, "fwd_qb") == 0) {
-    if (value < 0 || value > 2) return fail(FBA_ERR_INVALID, "fwd_qb must be 0..2, got %d", value);
-    g_fwd_qb.store(value);
-    return FBA_OK;
-  }
   return fail(FBA_ERR_INVALID, "unknown option '%s'", name);
 }
 
@@ -111,65 +104,66 @@ static int fill_bwd(fba::BwdParams& p, const Shape& s) {
   return FBA_OK;
 }
 
-int32_t fba_bwd_delta(const void* o, const void* d_o, float* delta, int64_t rows, int32_t head_dim, void* hip_stream) {
+int32_t fba_bwd_stats(const void* o, const void* d_o, const float* lse, float* stats, int64_t rows, int32_t head_dim,
+                      void* hip_stream) {
   if (head_dim != 128) return fail(FBA_ERR_INVALID, "head_dim must be 128, got %d", head_dim);
-  if (rows < 0) return fail(FBA_ERR_INVALID, "rows must be non-negative");
+  if (rows < 0 || rows >= (1LL << 30)) return fail(FBA_ERR_INVALID, "rows must be in [0, 2^30)");
   if (int rc = check_ptrs({{"o", o}, {"d_o", d_o}})) return rc;
-  if (!delta) return fail(FBA_ERR_INVALID, "delta is null");
-  hipError_t e = fba::launch_bwd_delta((const __bf16*)o, (const __bf16*)d_o, delta, rows, (hipStream_t)hip_stream);
-  return e == hipSuccess ? FBA_OK : hip_fail(e, "delta launch");
+  if (!lse || !stats) return fail(FBA_ERR_INVALID, "null pointer argument");
+  hipError_t e = fba::launch_bwd_stats((const __bf16*)o, (const __bf16*)d_o, lse, stats, rows, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "stats launch");
 }
 
-int32_t fba_bwd_dq(const void* q, const void* k, const void* v, const void* d_o, const float* lse, const float* delta,
-                   void* dq, const int32_t* q_cnt, const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq,
-                   int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,
-                   void* hip_stream) {
+int32_t fba_bwd_dq(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dq,
+                   const int32_t* q_cnt, const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
+                   int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"d_o", d_o}, {"dq", dq}})) return rc;
-  if (!lse || !delta || !q_cnt || !q_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
+  if (!stats || !q_cnt || !q_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
   if (q_block % 128 != 0)
     return fail(FBA_ERR_UNSUPPORTED, "dq: q_block (%d) must be a multiple of 128 in this build", q_block);
   fba::BwdParams p{};
   fill_bwd(p, s);
   p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.d_o = (const __bf16*)d_o;
-  p.lse = lse; p.delta = delta; p.dq = (__bf16*)dq; p.q_cnt = q_cnt; p.q_idx = q_idx;
+  p.stats = stats; p.dq = (__bf16*)dq; p.q_cnt = q_cnt; p.q_idx = q_idx;
   hipError_t e = fba::launch_bwd_dq(p, (hipStream_t)hip_stream);
   return e == hipSuccess ? FBA_OK : hip_fail(e, "dq launch");
 }
 
-int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* lse, const float* delta,
-                     void* dk, void* dv, const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B,
-                     int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block,
-                     int32_t k_block, void* hip_stream) {
+int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,
+                     const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
+                     int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"d_o", d_o}, {"dk", dk}, {"dv", dv}})) return rc;
-  if (!lse || !delta || !k_cnt || !k_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
+  if (!stats || !k_cnt || !k_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
   if (k_block % 128 != 0)
     return fail(FBA_ERR_UNSUPPORTED, "dkdv: k_block (%d) must be a multiple of 128 in this build", k_block);
-  if (q_block % 64 != 0)
-    return fail(FBA_ERR_UNSUPPORTED, "dkdv: q_block (%d) must be a multiple of 64 in this build", q_block);
+  if (q_block % 128 != 0)
+    return fail(FBA_ERR_UNSUPPORTED, "dkdv: q_block (%d) must be a multiple of 128 in this build", q_block);
+  if ((int64_t)B * Hq * Sq >= (1LL << 30)) return fail(FBA_ERR_INVALID, "B*Hq*Sq must be below 2^30");
   fba::BwdParams p{};
   fill_bwd(p, s);
   p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.d_o = (const __bf16*)d_o;
-  p.lse = lse; p.delta = delta; p.dk = (__bf16*)dk; p.dv = (__bf16*)dv; p.k_cnt = k_cnt; p.k_idx = k_idx;
+  p.stats = stats; p.dk = (__bf16*)dk; p.dv = (__bf16*)dv; p.k_cnt = k_cnt; p.k_idx = k_idx;
   hipError_t e = fba::launch_bwd_dkdv(p, (hipStream_t)hip_stream);
   return e == hipSuccess ? FBA_OK : hip_fail(e, "dkdv launch");
 }
 
 int32_t fba_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
-                float* delta, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
+                float* stats, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
                 const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
                 int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
-  if (int rc = fba_bwd_delta(o, d_o, delta, (int64_t)B * Hq * Sq, head_dim, hip_stream)) return rc;
-  if (int rc = fba_bwd_dkdv(q, k, v, d_o, lse, delta, dk, dv, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block,
-                            k_block, hip_stream))
+  if (q_block % 128 != 0 || k_block % 128 != 0)
+    return fail(FBA_ERR_UNSUPPORTED, "backward: q_block (%d) and k_block (%d) must be multiples of 128 in this build", q_block, k_block);
+  if (int rc = fba_bwd_stats(o, d_o, lse, stats, (int64_t)B * Hq * Sq, head_dim, hip_stream)) return rc;
+  if (int rc = fba_bwd_dkdv(q, k, v, d_o, stats, dk, dv, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block,
+                            hip_stream))
     return rc;
-  return fba_bwd_dq(q, k, v, d_o, lse, delta, dq, q_cnt, q_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block,
-                    hip_stream);
+  return fba_bwd_dq(q, k, v, d_o, stats, dq, q_cnt, q_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream);
 }
 
 }  // extern "C"

@@ -1,0 +1,215 @@
+// Backward, dK and dV: gfx950, head_dim 128, bf16 in / fp32 accumulate / bf16 out, no atomics.
+//
+// With P = exp(S/sqrt(D) - LSE), delta = rowsum(dO o O), dP = dO V^T, dS = P o (dP - delta) / sqrt(D):
+//   dV = P^T dO,  dK = dS^T Q                   (reference: flex_block_attn_h100.cu:498-537)
+// The reference accumulates dK and dV per CTA and adds them into fp32 buffers with reducing stores (:556, :566).  Here a
+// key-major kernel owns its dK / dV rows: it walks the per-key-block lists of every query head of the GQA group and
+// writes each output element once.
+//
+// Work-group = 128 key rows of one (batch, kv head), wave = 32 keys, lane = key:
+//   S = Q K^T, dP = dO V^T             A = Q / dO slab rows from LDS (128-bit fetches), B = K / V in registers
+//   P = exp2(c S - lse2[q]),  dS = P o (dP - delta[q])          (lse2, delta per accumulator row, read from LDS)
+//   dV^T += dO^T P,  dK^T += Q^T dS    A = dO / Q slab through transposing LDS fetches, B = P / dS packed to bf16
+// Software pipeline over 32-query slabs: while the VALU turns (S_t, dP_t) into P_t and dS_t, the matrix pipe computes
+// S_{t+1} and dP_{t+1}; the dV / dK updates of slab t follow.  Q, dO and the two statistics travel global -> LDS
+// directly into a ring of four (Q | dO | lse2 | delta) buffers; slab t+4 is requested when slab t is dead.
+#include <type_traits>
+
+#include "fba_common.h"
+#include "fba_kernels.h"
+
+namespace fba {
+
+namespace {
+
+constexpr int kSlab = 32;
+constexpr int kSlabBytes = kSlab * kRowBytes;       // 8 KiB
+constexpr int kStatBytes = 2 * kSlab * 4;           // lse2[32] | delta[32]
+constexpr int kStageBytes = 2 * kSlabBytes + kStatBytes;
+constexpr int kRing = 4;
+
+template <int N>
+using IC = std::integral_constant<int, N>;
+
+}  // namespace
+
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kernel(const BwdParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];  // ring [4] of (Q slab | dO slab | lse2 | delta)
+  constexpr int TK = 128;
+
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int item = xcd_remap(blockIdx.x, p.items_per_xcd);
+  if (item >= p.num_items) return;
+  const int tiles_per_head = p.Skv / TK;
+  const int bhk = item / tiles_per_head;
+  const int kt = item - bhk * tiles_per_head;
+  const int b = bhk / p.Hkv, hkv = bhk - b * p.Hkv;
+  const int group = p.Hq / p.Hkv;
+  const int kblk = (kt * TK) / p.k_block;
+
+  // K and V as B operands: lane holds key row l32, d = 16 ks + 8 h .. +7
+  const int64_t krow0 = (int64_t)bhk * p.Skv + (int64_t)kt * TK + wave * 32;
+  bf16x8 kreg[8], vreg[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    kreg[ks] = *reinterpret_cast<const bf16x8*>(p.k + (krow0 + l32) * kHeadDim + 16 * ks + 8 * h);
+    vreg[ks] = *reinterpret_cast<const bf16x8*>(p.v + (krow0 + l32) * kHeadDim + 16 * ks + 8 * h);
+  }
+
+  const int nsub = p.q_block / kSlab;
+  auto list_row = [&](int g) -> int64_t {
+    const int64_t bh = (int64_t)b * p.Hq + hkv * group + g;
+    return (p.mask_bh == 1 ? 0 : bh) * p.nK + kblk;
+  };
+  int nsteps = 0;
+  for (int g = 0; g < group; ++g) nsteps += p.k_cnt[list_row(g)];
+  nsteps *= nsub;
+
+  RowMajorOffsets rm;
+  rm.init(lane);
+  TransposedOffsets tr;
+  tr.init(lane);
+  SlabDma dma;
+  dma.init(wave, lane);
+  const uint32_t ring_dst = lds_addr(smem);
+  const int64_t rows_total = (int64_t)p.B * p.Hq * p.Sq;
+  // statistics copy: lanes 0..31 fetch lse2[row0 + l], lanes 32..63 fetch delta[row0 + l - 32]
+  const uint32_t stat_off = (uint32_t)((lane >> 5) * rows_total * 4 + (lane & 31) * 4);
+  const float c = p.scale_log2e;
+
+  f32x16 acc_k[4], acc_v[4];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { acc_k[mb][r] = 0.f; acc_v[mb][r] = 0.f; }
+
+  // Cursor over (query head of the group, list entry, slab): first query row of the next slab to request.
+  const char* qbase = reinterpret_cast<const char*>(p.q);
+  const char* dobase = reinterpret_cast<const char*>(p.d_o);
+  const char* stbase = reinterpret_cast<const char*>(p.stats);
+  int g_cur = -1, e_cur = 0, cnt_cur = 0, rem = 1;
+  ConstIdx idx_cur = nullptr;
+  int64_t row_next = 0, head_row0 = 0;
+  auto next_block = [&]() {  // position row_next on the first row of the next listed query block, if any
+    ++e_cur;
+    while (e_cur >= cnt_cur) {
+      if (++g_cur >= group) return;
+      const int64_t lr = list_row(g_cur);
+      cnt_cur = p.k_cnt[lr];
+      idx_cur = const_idx(p.k_idx + lr * p.nQ);
+      head_row0 = ((int64_t)b * p.Hq + hkv * group + g_cur) * p.Sq;
+      e_cur = 0;
+    }
+    row_next = head_row0 + (int64_t)idx_cur[e_cur] * p.q_block;
+    rem = nsub;
+  };
+  auto copy_next = [&](int ring) {
+    const uint32_t dst = ring_dst + ring * kStageBytes;
+    dma.copy(dst, qbase + row_next * kRowBytes);
+    dma.copy(dst + kSlabBytes, dobase + row_next * kRowBytes);
+    dma4(dst + 2 * kSlabBytes, stbase + row_next * 4, stat_off);  // every wave copies the same 256 bytes
+    if (--rem == 0) next_block(); else row_next += kSlab;
+  };
+
+  // S and dP of one slab: 16 MFMAs, the two chains interleaved
+  auto scores = [&](const char* stage, f32x16& s, f32x16& dp) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      s = mfma32(lds_read_b128(stage, rm.rd[ks]), kreg[ks], s);
+      dp = mfma32(lds_read_b128(stage + kSlabBytes, rm.rd[ks]), vreg[ks], dp);
+    }
+  };
+
+  if (nsteps > 0) {
+    e_cur = -1;
+    next_block();
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (j < nsteps) copy_next(j);
+    wait_vmem<0>();
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) { pin(kreg[ks]); pin(vreg[ks]); }
+    f32x16 s_cur, dp_cur;
+    scores(smem, s_cur, dp_cur);
+
+    // step t (t % 4 == R): P_t, dS_t from (S_t, dP_t) | S_{t+1}, dP_{t+1} from slab t+1 | dV += dO_t^T P_t, dK += Q_t^T dS_t
+    auto step = [&](auto ring_c, int t) {
+      constexpr int R = decltype(ring_c)::value;
+      const char* stage = smem + R * kStageBytes;
+      f32x16 s_nxt, dp_nxt;
+      scores(smem + ((R + 1) & 3) * kStageBytes, s_nxt, dp_nxt);  // past the last slab: stale data, unused
+      const float* st_lds = reinterpret_cast<const float*>(stage + 2 * kSlabBytes);
+      // accumulator element 4g + e of half-wave h is query row 8g + 4h + e of the slab
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 l4 = *reinterpret_cast<const f32x4*>(st_lds + 8 * g + 4 * h);
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(st_lds + kSlab + 8 * g + 4 * h);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float pv = fast_exp2(__builtin_fmaf(s_cur[4 * g + e], c, -l4[e]));
+          s_cur[4 * g + e] = pv;
+          dp_cur[4 * g + e] = pv * (dp_cur[4 * g + e] - d4[e]);
+        }
+      }
+      bf16x8 pk[2], dsk[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        pk[j] = pack8(s_cur[8 * j + 0], s_cur[8 * j + 1], s_cur[8 * j + 2], s_cur[8 * j + 3], s_cur[8 * j + 4],
+                      s_cur[8 * j + 5], s_cur[8 * j + 6], s_cur[8 * j + 7]);
+        dsk[j] = pack8(dp_cur[8 * j + 0], dp_cur[8 * j + 1], dp_cur[8 * j + 2], dp_cur[8 * j + 3], dp_cur[8 * j + 4],
+                       dp_cur[8 * j + 5], dp_cur[8 * j + 6], dp_cur[8 * j + 7]);
+      }
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) {
+          const int roff = 16 * j * kRowBytes;
+          const bf16x8 adv = cat(lds_read_tr(stage + kSlabBytes, tr.rd[mb][0] + roff), lds_read_tr(stage + kSlabBytes, tr.rd[mb][1] + roff));
+          acc_v[mb] = mfma32(adv, pk[j], acc_v[mb]);
+          const bf16x8 adk = cat(lds_read_tr(stage, tr.rd[mb][0] + roff), lds_read_tr(stage, tr.rd[mb][1] + roff));
+          acc_k[mb] = mfma32(adk, dsk[j], acc_k[mb]);
+        }
+      s_cur = s_nxt;
+      dp_cur = dp_nxt;
+      // slab t+2 must have landed (first read in step t+1); the five copies of slab t+3 may still fly
+      if (t + 3 < nsteps) wait_vmem<5>(); else wait_vmem<0>();
+      __syncthreads();
+      if (t + 4 < nsteps) copy_next(R);
+    };
+    for (int t = 0; t < nsteps; t += 4) {  // nsteps is a multiple of 4
+      step(IC<0>{}, t);
+      step(IC<1>{}, t + 1);
+      step(IC<2>{}, t + 2);
+      step(IC<3>{}, t + 3);
+    }
+  }
+
+  __bf16* dkrow = p.dk + (krow0 + l32) * kHeadDim;
+  __bf16* dvrow = p.dv + (krow0 + l32) * kHeadDim;
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const bf16x4 kv = pack4(acc_k[mb][4 * g + 0] * p.scale, acc_k[mb][4 * g + 1] * p.scale, acc_k[mb][4 * g + 2] * p.scale,
+                              acc_k[mb][4 * g + 3] * p.scale);
+      const bf16x4 vv = pack4(acc_v[mb][4 * g + 0], acc_v[mb][4 * g + 1], acc_v[mb][4 * g + 2], acc_v[mb][4 * g + 3]);
+      *reinterpret_cast<bf16x4*>(dkrow + 32 * mb + 8 * g + 4 * h) = kv;
+      *reinterpret_cast<bf16x4*>(dvrow + 32 * mb + 8 * g + 4 * h) = vv;
+    }
+}
+
+hipError_t launch_bwd_dkdv(BwdParams p, hipStream_t stream) {
+  constexpr int kSmem = kRing * kStageBytes;
+  p.num_items = p.B * p.Hkv * (p.Skv / 128);
+  p.items_per_xcd = (p.num_items + kNumXcd - 1) / kNumXcd;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(dkdv_kernel, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
+  return hipGetLastError();
+}
+
+}  // namespace fba

@@ -1,0 +1,204 @@
+// Backward, dQ: gfx950, head_dim 128, bf16 in / fp32 accumulate / bf16 out, no atomics.
+//
+// With P = exp(S/sqrt(D) - LSE), delta = rowsum(dO o O), dP = dO V^T, dS = P o (dP - delta) / sqrt(D):
+//   dQ = dS K                                   (reference: flex_block_attn_h100.cu:498-529, :750-753)
+// The reference forms dQ inside its key-major kernel and adds it into an fp32 buffer with reducing stores
+// (:707-708).  Here a query-major kernel owns its dQ rows: it walks the per-query-block lists exactly like the forward
+// kernel and recomputes S and dP.
+//
+// Work-group = 128 query rows, wave = 32 rows, lane = query row (everything transposed, as in the forward kernel):
+//   S^T = K Q^T, dP^T = V dO^T         A = K / V slab rows from LDS (128-bit fetches), B = Q / dO in registers
+//   dS^T = exp2(c S^T - lse2) o (dP^T - delta)
+//   dQ^T += K^T dS^T                   A = K slab through transposing LDS fetches, B = dS^T packed to bf16
+// Software pipeline over 32-key slabs: while the VALU turns (S_t, dP_t) into dS_t, the matrix pipe computes S_{t+1} and
+// dP_{t+1}; the dQ update with dS_t follows.  K and V slabs travel global -> LDS directly into a ring of four
+// (K | V) buffers; slab t+4 is requested when slab t is dead, three steps before its first use.
+#include <type_traits>
+
+#include "fba_common.h"
+#include "fba_kernels.h"
+
+// 1: S and dP of slab t+1 are computed during step t (needs both score sets live: more than 256 registers, one wave
+// per SIMD); 0: every step computes its own scores and two waves per SIMD overlap each other.
+#ifndef FBA_DQ_PIPELINED
+#define FBA_DQ_PIPELINED 0
+#endif
+
+namespace fba {
+
+namespace {
+
+constexpr int kSlab = 32;
+constexpr int kSlabBytes = kSlab * kRowBytes;  // 8 KiB
+constexpr int kPairBytes = 2 * kSlabBytes;     // K slab | V slab
+constexpr int kRing = 4;
+
+template <int N>
+using IC = std::integral_constant<int, N>;
+
+}  // namespace
+
+#if FBA_DQ_PIPELINED
+#define FBA_DQ_OCCUPANCY
+#else
+#define FBA_DQ_OCCUPANCY , amdgpu_waves_per_eu(2, 2)
+#endif
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256) FBA_DQ_OCCUPANCY)) void dq_kernel(const BwdParams p) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];  // ring [4] of (K slab | V slab)
+  constexpr int TQ = 128;
+
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int item = xcd_remap(blockIdx.x, p.items_per_xcd);
+  if (item >= p.num_items) return;
+  const int tiles_per_head = p.Sq / TQ;
+  const int bh = item / tiles_per_head;
+  const int qt = item - bh * tiles_per_head;
+  const int b = bh / p.Hq, hq = bh - b * p.Hq;
+  const int hkv = hq / (p.Hq / p.Hkv);
+
+  const int64_t qrow0 = (int64_t)bh * p.Sq + (int64_t)qt * TQ + wave * 32;
+  const char* kp = reinterpret_cast<const char*>(p.k + ((int64_t)(b * p.Hkv + hkv) * p.Skv) * kHeadDim);
+  const char* vp = reinterpret_cast<const char*>(p.v + ((int64_t)(b * p.Hkv + hkv) * p.Skv) * kHeadDim);
+
+  const int qblk = (qt * TQ) / p.q_block;
+  const int64_t mrow = (p.mask_bh == 1 ? 0 : (int64_t)bh) * p.nQ + qblk;
+  const int cnt = p.q_cnt[mrow];
+  const ConstIdx idx = const_idx(p.q_idx + mrow * p.nK);
+  const int nsub = p.k_block / kSlab;
+  const int nsteps = cnt * nsub;
+
+  // Q and dO as B operands: lane holds row l32, d = 16 ks + 8 h .. +7
+  bf16x8 qreg[8], doreg[8];
+#pragma unroll
+  for (int ks = 0; ks < 8; ++ks) {
+    qreg[ks] = *reinterpret_cast<const bf16x8*>(p.q + (qrow0 + l32) * kHeadDim + 16 * ks + 8 * h);
+    doreg[ks] = *reinterpret_cast<const bf16x8*>(p.d_o + (qrow0 + l32) * kHeadDim + 16 * ks + 8 * h);
+  }
+  const int64_t rows_total = (int64_t)p.B * p.Hq * p.Sq;
+  const float lse2 = p.stats[qrow0 + l32];
+  const float dlt = p.stats[rows_total + qrow0 + l32];
+  const float c = p.scale_log2e;
+
+  RowMajorOffsets rm;
+  rm.init(lane);
+  TransposedOffsets tr;
+  tr.init(lane);
+  SlabDma dma;
+  dma.init(wave, lane);
+  const uint32_t ring_dst = lds_addr(smem);
+
+  f32x16 acc[4];
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[mb][r] = 0.f;
+
+  // slab source offsets in list order; the list entry of the following key block is read one block ahead
+  const int64_t block_bytes = (int64_t)p.k_block * kRowBytes;
+  int e_next = 1, rem = nsub;
+  int64_t src_off = cnt > 0 ? idx[0] * block_bytes : 0;
+  int blk_next = cnt > 1 ? idx[1] : 0;
+  auto copy_next = [&](int ring) {
+    dma.copy(ring_dst + ring * kPairBytes, kp + src_off);
+    dma.copy(ring_dst + ring * kPairBytes + kSlabBytes, vp + src_off);
+    if (--rem == 0) {
+      rem = nsub;
+      src_off = blk_next * block_bytes;
+      ++e_next;
+      blk_next = e_next < cnt ? idx[e_next] : 0;
+    } else {
+      src_off += kSlabBytes;
+    }
+  };
+
+  // S^T and dP^T of one slab: 16 MFMAs, the two chains interleaved
+  auto scores = [&](const char* pair, f32x16& s, f32x16& dp) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      s = mfma32(lds_read_b128(pair, rm.rd[ks]), qreg[ks], s);
+      dp = mfma32(lds_read_b128(pair + kSlabBytes, rm.rd[ks]), doreg[ks], dp);
+    }
+  };
+
+  if (nsteps > 0) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      if (j < nsteps) copy_next(j);
+    wait_vmem<0>();
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) { pin(qreg[ks]); pin(doreg[ks]); }
+#if FBA_DQ_PIPELINED
+    f32x16 s_cur, dp_cur;
+    scores(smem, s_cur, dp_cur);
+#endif
+
+    // step t (t % 4 == R): dS_t from (S_t, dP_t) | S_{t+1}, dP_{t+1} from slab t+1 | dQ += K_t^T dS_t
+    auto step = [&](auto ring_c, int t) {
+      constexpr int R = decltype(ring_c)::value;
+#if FBA_DQ_PIPELINED
+      f32x16 s_nxt, dp_nxt;
+      scores(smem + ((R + 1) & 3) * kPairBytes, s_nxt, dp_nxt);  // past the last slab: stale data, unused
+#else
+      f32x16 s_cur, dp_cur;
+      scores(smem + R * kPairBytes, s_cur, dp_cur);
+#endif
+      bf16x8 dsk[2];
+#pragma unroll
+      for (int r = 0; r < 16; ++r) s_cur[r] = fast_exp2(__builtin_fmaf(s_cur[r], c, -lse2)) * (dp_cur[r] - dlt);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        dsk[j] = pack8(s_cur[8 * j + 0], s_cur[8 * j + 1], s_cur[8 * j + 2], s_cur[8 * j + 3], s_cur[8 * j + 4],
+                       s_cur[8 * j + 5], s_cur[8 * j + 6], s_cur[8 * j + 7]);
+      const char* k_t = smem + R * kPairBytes;
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) {
+          const int roff = 16 * j * kRowBytes;
+          const bf16x8 a = cat(lds_read_tr(k_t, tr.rd[mb][0] + roff), lds_read_tr(k_t, tr.rd[mb][1] + roff));
+          acc[mb] = mfma32(a, dsk[j], acc[mb]);
+        }
+#if FBA_DQ_PIPELINED
+      s_cur = s_nxt;
+      dp_cur = dp_nxt;
+#endif
+      // slab t+2 must have landed (first read in step t+1); the four copies of slab t+3 may still fly
+      if (t + 3 < nsteps) wait_vmem<4>(); else wait_vmem<0>();
+      __syncthreads();
+      if (t + 4 < nsteps) copy_next(R);
+    };
+    for (int t = 0; t < nsteps; t += 4) {  // nsteps is even
+      step(IC<0>{}, t);
+      step(IC<1>{}, t + 1);
+      if (t + 2 >= nsteps) break;
+      step(IC<2>{}, t + 2);
+      step(IC<3>{}, t + 3);
+    }
+  }
+
+  __bf16* orow = p.dq + (qrow0 + l32) * kHeadDim;
+#pragma unroll
+  for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const bf16x4 ov = pack4(acc[mb][4 * g + 0] * p.scale, acc[mb][4 * g + 1] * p.scale, acc[mb][4 * g + 2] * p.scale,
+                              acc[mb][4 * g + 3] * p.scale);
+      *reinterpret_cast<bf16x4*>(orow + 32 * mb + 8 * g + 4 * h) = ov;
+    }
+}
+
+hipError_t launch_bwd_dq(BwdParams p, hipStream_t stream) {
+  constexpr int kSmem = kRing * kPairBytes;
+  p.num_items = p.B * p.Hq * (p.Sq / 128);
+  p.items_per_xcd = (p.num_items + kNumXcd - 1) / kNumXcd;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(dq_kernel, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
+  return hipGetLastError();
+}
+
+}  // namespace fba

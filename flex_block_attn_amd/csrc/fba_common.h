@@ -150,9 +150,38 @@ FBA_DEVICE void dma16(uint32_t lds_base, const char* gbase, uint32_t lane_off) {
                : "m0");
 }
 
-// Wait until at most N vector-memory loads are outstanding (N < 16).
+// Same for 4 bytes per lane (lane l's dword lands at lds_base + 4 l).
+FBA_DEVICE void dma4(uint32_t lds_base, const char* gbase, uint32_t lane_off) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+               :
+               : "s"(lds_base), "v"(lane_off), "s"(gbase)
+               : "m0");
+}
+
+// Wait until at most N vector-memory loads are outstanding (N < 64; the counter's two high bits sit in bits 15:14).
 template <int N>
-FBA_DEVICE void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70 | N); }
+FBA_DEVICE void wait_vmem() { __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14)); }
+
+// Direct copy of a 32-row slab (32 x 128 bf16, 8 KiB) from global memory into a swizzled LDS tile by the 4 waves of a
+// work-group.  A wave-level copy fills 1 KiB = 4 rows; wave w owns rows 8w .. 8w+7 (two copies).  Lane l lands in row
+// 8w + 4g + l/16, chunk slot l%16, so it fetches chunk (l%16) ^ swz(row) of that row.
+struct SlabDma {
+  uint32_t off[2];
+  uint32_t wave_dst;  // byte offset of the wave's rows inside a slab
+  FBA_DEVICE void init(int wave, int lane) {
+#pragma unroll
+    for (int g = 0; g < 2; ++g) {
+      const int row = 8 * wave + 4 * g + (lane >> 4);
+      off[g] = (uint32_t)(row * kRowBytes + (((lane & 15) ^ swz(row)) << 4));
+    }
+    wave_dst = (uint32_t)(wave * 8 * kRowBytes);
+  }
+  // slab_lds: LDS address of the slab buffer; src: global address of the slab's first row (both wave-uniform)
+  FBA_DEVICE void copy(uint32_t slab_lds, const char* src) const {
+    dma16(slab_lds + wave_dst, src, off[0]);
+    dma16(slab_lds + wave_dst + 4 * kRowBytes, src, off[1]);
+  }
+};
 
 // Per-lane LDS offsets for row-major A/B operand fetches of a 32-row slab: rd[ks] addresses row (lane % 32),
 // chunk 2*ks + lane/32.  Add 32*kRowBytes per further slab (rows stay congruent mod 16, so swz is unchanged).

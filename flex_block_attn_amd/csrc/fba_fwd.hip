@@ -146,18 +146,12 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 #pragma unroll
     for (int r = 0; r < 16; ++r) st.acc_o[mb][r] = 0.f;
 
-  // Slab copies.  A wave-level copy fills 1 KiB = 4 rows of a slab; wave w owns rows 8w .. 8w+7 (two copies).  Lane l
-  // lands in row 4g + l/16, chunk slot l%16, so it must fetch chunk (l%16) ^ swz(row) of that row.
-  uint32_t dma_off[2];
-#pragma unroll
-  for (int g = 0; g < 2; ++g) {
-    const int row = 8 * wave + 4 * g + (lane >> 4);
-    dma_off[g] = (uint32_t)(row * kRowBytes + (((lane & 15) ^ swz(row)) << 4));
-  }
+  SlabDma dma;
+  dma.init(wave, lane);
   char* const k_lds = smem;
   char* const v_lds = smem + kRing * kSlabBytes;
-  const uint32_t k_dst = lds_addr(k_lds) + wave * 8 * kRowBytes;
-  const uint32_t v_dst = lds_addr(v_lds) + wave * 8 * kRowBytes;
+  const uint32_t k_dst = lds_addr(k_lds);
+  const uint32_t v_dst = lds_addr(v_lds);
 
   // Slab source offsets, in list order.  The list entry of the following key block is read one block ahead, so that
   // the scalar load is off the critical path.  V requests trail K requests by two slabs and reuse their offsets.
@@ -177,10 +171,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     }
     return off;
   };
-  auto copy_slab = [&](uint32_t dst, const char* src) {
-    dma16(dst, src, dma_off[0]);
-    dma16(dst + 4 * kRowBytes, src, dma_off[1]);
-  };
+  auto copy_slab = [&](uint32_t dst, const char* src) { dma.copy(dst, src); };
 
   if (nsteps > 0) {
     // prologue: K_0..K_3 and V_0..V_2 requested, S_0 computed, then K_4 into the buffer of K_0

@@ -30,8 +30,7 @@ struct BwdParams {
   const __bf16* k;
   const __bf16* v;
   const __bf16* d_o;
-  const float* lse;
-  const float* delta;  // [B, Hq, Sq]
+  const float* stats;  // [2, B, Hq, Sq]: lse * log2(e), then delta = rowsum(dO o O)
   __bf16* dq;
   __bf16* dk;
   __bf16* dv;
@@ -49,7 +48,7 @@ struct BwdParams {
 hipError_t launch_mask_compact(const uint8_t* mask, int64_t mask_bh, int nQ, int nK, int32_t* q_cnt, int32_t* q_idx,
                                int32_t* k_cnt, int32_t* k_idx, hipStream_t stream);
 hipError_t launch_fwd(FwdParams p, hipStream_t stream);
-hipError_t launch_bwd_delta(const __bf16* o, const __bf16* d_o, float* delta, int64_t rows, hipStream_t stream);
+hipError_t launch_bwd_stats(const __bf16* o, const __bf16* d_o, const float* lse, float* stats, int64_t rows, hipStream_t stream);
 hipError_t launch_bwd_dq(BwdParams p, hipStream_t stream);
 hipError_t launch_bwd_dkdv(BwdParams p, hipStream_t stream);
 

@@ -54,11 +54,13 @@ hipError_t launch_mask_compact(const uint8_t* mask, int64_t mask_bh, int nQ, int
   return hipGetLastError();
 }
 
-// delta[r] = sum_c dO[r, c] * O[r, c] in fp32 (reference: bwd_attend_prep_ker, flex_block_attn_h100.cu:375-379).
-// 16 lanes per row (16 bytes of each operand per lane), 16 rows per 256-thread work-group pass.
-__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void bwd_delta_kernel(const __bf16* __restrict__ o,
+// Backward statistics, one pass over O and dO: stats[r] = lse[r] * log2(e) and stats[rows + r] = delta[r] =
+// sum_c dO[r, c] * O[r, c] in fp32 (reference: bwd_attend_prep_ker, flex_block_attn_h100.cu:375-379).  The backward
+// kernels exponentiate in base 2, hence the pre-scaled LSE.  16 lanes per row (16 bytes of each operand per lane).
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void bwd_stats_kernel(const __bf16* __restrict__ o,
                                                                                         const __bf16* __restrict__ d_o,
-                                                                                        float* __restrict__ delta, int64_t rows) {
+                                                                                        const float* __restrict__ lse,
+                                                                                        float* __restrict__ stats, int64_t rows) {
   const int sub = threadIdx.x & 15;
   for (int64_t r = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4); r < rows; r += (int64_t)gridDim.x * 16) {
     const bf16x8 a = *reinterpret_cast<const bf16x8*>(o + r * kHeadDim + sub * 8);
@@ -70,15 +72,18 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void bwd_delta
     acc += __shfl_xor(acc, 4);
     acc += __shfl_xor(acc, 2);
     acc += __shfl_xor(acc, 1);
-    if (sub == 0) delta[r] = acc;
+    if (sub == 0) {
+      stats[r] = lse[r] * 1.4426950408889634f;
+      stats[rows + r] = acc;
+    }
   }
 }
 
-hipError_t launch_bwd_delta(const __bf16* o, const __bf16* d_o, float* delta, int64_t rows, hipStream_t stream) {
+hipError_t launch_bwd_stats(const __bf16* o, const __bf16* d_o, const float* lse, float* stats, int64_t rows, hipStream_t stream) {
   if (rows <= 0) return hipSuccess;
   int64_t blocks = (rows + 15) / 16;
   if (blocks > 65536) blocks = 65536;
-  hipLaunchKernelGGL(bwd_delta_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, o, d_o, delta, rows);
+  hipLaunchKernelGGL(bwd_stats_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, o, d_o, lse, stats, rows);
   return hipGetLastError();
 }
 

@@ -160,10 +160,10 @@ def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists)
     dq = torch.empty_like(q)
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)
-    delta = torch.empty((B, Hq, Sq), dtype=torch.float32, device=q.device)
+    stats = torch.empty((2, B, Hq, Sq), dtype=torch.float32, device=q.device)
     with torch.cuda.device(q.device):
         _lib.call(
-            "fba_bwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(delta), _ptr(dq), _ptr(dk), _ptr(dv),
+            "fba_bwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), _ptr(dq), _ptr(dk), _ptr(dv),
             _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), lists.mask_bh,
             B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size, _stream(),
         )

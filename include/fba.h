@@ -65,29 +65,27 @@ int32_t fba_fwd(const void* q, const void* k, const void* v, void* o, float* lse
 /*
  * Backward, three stream-ordered launches.  Replaces attn_backward (attn.cpp:30,
  * flex_block_attn_h100.cu:1009-1267): bwd_attend_prep_ker (:324-389) and bwd_attend_ker (:572-802).
- *   delta    [B, Hq, Sq] fp32 workspace, written by the call (rowsum(dO o O))
+ *   stats    [2, B, Hq, Sq] fp32 workspace written by the call: lse * log2(e), then delta = rowsum(dO o O)
  *   dq       [B, Hq, Sq, 128] bf16;  dk, dv [B, Hkv, Skv, 128] bf16 (summed over the query heads of a GQA group)
  * Every output element is written exactly once; no buffer needs clearing beforehand.
  */
 int32_t fba_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
-                float* delta, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
+                float* stats, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
                 const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
                 int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
 
-/* The three stages of fba_bwd, separately (same arguments, for profiling one kernel at a time). */
-int32_t fba_bwd_delta(const void* o, const void* d_o, float* delta, int64_t rows, int32_t head_dim, void* hip_stream);
-int32_t fba_bwd_dq(const void* q, const void* k, const void* v, const void* d_o, const float* lse, const float* delta,
-                   void* dq, const int32_t* q_cnt, const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq,
-                   int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,
-                   void* hip_stream);
-int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* lse, const float* delta,
-                     void* dk, void* dv, const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B,
-                     int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block,
-                     int32_t k_block, void* hip_stream);
+/* The three stages of fba_bwd, separately (for profiling one kernel at a time); rows = B * Hq * Sq. */
+int32_t fba_bwd_stats(const void* o, const void* d_o, const float* lse, float* stats, int64_t rows, int32_t head_dim,
+                      void* hip_stream);
+int32_t fba_bwd_dq(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dq,
+                   const int32_t* q_cnt, const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
+                   int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,
+                     const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
+                     int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
 
 /*
- * Tuning knobs for experiments (process-wide).  Known names: "fwd_qb" (query rows per forward work-group in units
- * of 128; 0 = choose automatically).  Returns FBA_ERR_INVALID for an unknown name or value.
+ * Tuning knobs for experiments (process-wide).  No knob is defined at present; every name returns FBA_ERR_INVALID.
  */
 int32_t fba_set_option(const char* name, int32_t value);
 
