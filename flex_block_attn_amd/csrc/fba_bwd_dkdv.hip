@@ -62,8 +62,9 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
     const int64_t bh = (int64_t)b * p.Hq + hkv * group + g;
     return (p.mask_bh == 1 ? 0 : bh) * p.nK + kblk;
   };
+  const ConstIdx k_cnt = const_idx(p.k_cnt);
   int nsteps = 0;
-  for (int g = 0; g < group; ++g) nsteps += p.k_cnt[list_row(g)];
+  for (int g = 0; g < group; ++g) nsteps += k_cnt[list_row(g)];
   nsteps *= nsub;
 
   RowMajorOffsets rm;
@@ -96,7 +97,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
     while (e_cur >= cnt_cur) {
       if (++g_cur >= group) return;
       const int64_t lr = list_row(g_cur);
-      cnt_cur = p.k_cnt[lr];
+      cnt_cur = k_cnt[lr];
       idx_cur = const_idx(p.k_idx + lr * p.nQ);
       head_row0 = ((int64_t)b * p.Hq + hkv * group + g_cur) * p.Sq;
       e_cur = 0;

@@ -200,13 +200,14 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 
     bf16x8 p_prev[2];
 
-    // step t (t % 4 == R): softmax(S_t) | S_{t+1} = K_{t+1} Q^T | O += P_{t-1} V_{t-1}
+    // step t (t % 4 == R): O += P_{t-1} V_{t-1} | softmax(S_t) | S_{t+1} = K_{t+1} Q^T
     auto step = [&](auto ring_c, auto first_c, int t) {
       constexpr int R = decltype(ring_c)::value;
       constexpr bool kFirst = decltype(first_c)::value;
+      // P_{t-1} was formed against the reference m of step t-1, so it must reach O before step t may raise m
+      if constexpr (!kFirst) pv_half(st, v_lds + ((R + 3) & 3) * kSlabBytes, p_prev);
       softmax_reference(st, s_cur);
       const f32x16 s_nxt = qk_half(st, k_lds + ((R + 1) & 3) * kSlabBytes);  // past the last slab: stale data, unused
-      if constexpr (!kFirst) pv_half(st, v_lds + ((R + 3) & 3) * kSlabBytes, p_prev);
       softmax_exp(st, s_cur, p_prev);  // p_prev := P_t
       // P_t is only consumed after the barrier; without the pins its arithmetic sinks there, away from the MFMAs it is
       // meant to overlap with

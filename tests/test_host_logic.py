@@ -1,0 +1,179 @@
+"""Host-side checks that need no GPU: the C ABI loads and exports every declared symbol, argument validation fails the
+way the header says, the Python operator surface mirrors the reference's checks, and the mask helpers behave."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from flex_block_attn_amd import _lib
+
+    if not os.path.exists(_lib.LIB_PATH):
+        from flex_block_attn_amd import build
+
+        build.build_library()
+    return _lib
+
+
+def test_every_declared_symbol_is_exported(lib):
+    header = open(os.path.join(ROOT, "include", "fba.h")).read()
+    declared = set(re.findall(r"\b(fba_[a-z_0-9]+)\s*\(", header))
+    assert declared == set(lib.SIGNATURES), "include/fba.h and the ctypes table disagree"
+    handle = lib.load()
+    for name in declared:
+        assert getattr(handle, name) is not None
+    assert handle.fba_version() >= 1000
+
+
+def _null():
+    return ctypes.c_void_p(0)
+
+
+def _fake(addr=0x1000):
+    return ctypes.c_void_p(addr)
+
+
+def test_c_abi_argument_validation(lib):
+    h = lib.load()
+    f = _fake()
+    # fba_fwd(q,k,v,o,lse,q_cnt,q_idx, mask_bh, B,Hq,Hkv,Sq,Skv,D,q_block,k_block, stream)
+    ok_shape = (1, 1, 2, 2, 256, 256, 128, 128, 128)
+
+    def fwd(*shape, q=f):
+        return h.fba_fwd(q, f, f, f, f, f, f, *shape, _null())
+
+    bad = [
+        ((1, 1, 2, 2, 256, 256, 64, 128, 128), "head_dim"),
+        ((1, 1, 3, 2, 256, 256, 128, 128, 128), "multiple of Hkv"),
+        ((1, 1, 2, 2, 256, 256, 128, 24, 128), "q_block"),
+        ((1, 1, 2, 2, 256, 256, 128, 128, 96), "k_block"),
+        ((1, 1, 2, 2, 256, 384, 128, 128, 192), "divide"),
+        ((1, 1, 2, 2, 200, 256, 128, 128, 128), "Sq"),
+        ((1, 1, 2, 2, 256, 200, 128, 128, 128), "Skv"),
+        ((3, 1, 2, 2, 256, 256, 128, 128, 128), "mask_bh"),
+        ((1, 0, 2, 2, 256, 256, 128, 128, 128), "positive"),
+    ]
+    for shape, needle in bad:
+        assert fwd(*shape) == lib.FBA_ERR_INVALID, shape
+        assert needle in h.fba_last_error().decode(), (shape, h.fba_last_error())
+    assert fwd(*ok_shape, q=_null()) == lib.FBA_ERR_INVALID and b"q is null" in h.fba_last_error()
+    assert fwd(*ok_shape, q=_fake(0x1008)) == lib.FBA_ERR_INVALID and b"aligned" in h.fba_last_error()
+    # a shape the operator allows but no kernel variant covers yet is reported as such, not computed wrongly
+    assert fwd(1, 1, 2, 2, 256, 256, 128, 64, 128) == lib.FBA_ERR_UNSUPPORTED
+    assert b"q_block" in h.fba_last_error()
+    assert h.fba_mask_compact(f, 0, 4, 4, f, f, f, f, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_mask_compact(_null(), 1, 4, 4, f, f, f, f, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_bwd_stats(f, f, f, f, 16, 64, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_set_option(b"no_such_knob", 1) == lib.FBA_ERR_INVALID
+    with pytest.raises(lib.FbaError) as ei:
+        lib.call("fba_set_option", b"no_such_knob", 1)
+    assert ei.value.code == lib.FBA_ERR_INVALID and "no_such_knob" in ei.value.message
+
+
+def test_operator_surface_names():
+    import flex_block_attn
+    import flex_block_attn_amd as fba
+
+    for name in ("flex_block_attn_func", "_flex_block_attn_forward", "_flex_block_attn_backward"):
+        assert getattr(flex_block_attn, name) is getattr(fba, name)
+    import inspect
+
+    assert list(inspect.signature(fba.flex_block_attn_func).parameters) == ["q", "k", "v", "q_block_size", "kv_block_size", "block_mask"]
+    assert list(inspect.signature(fba._flex_block_attn_forward).parameters) == [
+        "q", "k", "v", "q_block_size", "kv_block_size", "block_mask", "small_block_mask", "use_small_block_mode"]
+    assert list(inspect.signature(fba._flex_block_attn_backward).parameters) == [
+        "q", "k", "v", "o", "lse", "do", "q_block_size", "kv_block_size", "block_mask", "small_block_mask", "use_small_block_mode"]
+
+
+def test_shape_rules_match_reference_asserts():
+    """Same conditions as flex_block_attn_interface.py:18-32, raised before anything touches a device."""
+    from flex_block_attn_amd.interface import _check_blocks
+
+    q = torch.zeros((1, 2, 768, 128), dtype=torch.bfloat16)
+    k = torch.zeros((1, 2, 768, 128), dtype=torch.bfloat16)
+    m = torch.ones((2, 2), dtype=torch.bool)
+    _check_blocks(q, k, 384, 384, m)
+    with pytest.raises(AssertionError, match="divisible by 16"):
+        _check_blocks(q, k, 24, 384, m)
+    with pytest.raises(AssertionError, match="divisible by 64"):
+        _check_blocks(q, k, 384, 96, m)
+    with pytest.raises(AssertionError, match="vice versa"):
+        _check_blocks(q, k, 48, 64, torch.ones((16, 12), dtype=torch.bool))
+    with pytest.raises(AssertionError, match="q_seq_len"):
+        _check_blocks(q, k, 512, 256, m)
+    with pytest.raises(AssertionError, match="q_block_num"):
+        _check_blocks(q, k, 384, 384, torch.ones((3, 2), dtype=torch.bool))
+    with pytest.raises(AssertionError, match="kv_block_num"):
+        _check_blocks(q, k, 384, 384, torch.ones((2, 3), dtype=torch.bool))
+    with pytest.raises(ValueError, match="2 or 4"):
+        _check_blocks(q, k, 384, 384, torch.ones((1, 2, 2), dtype=torch.bool))
+    with pytest.raises(ValueError, match="4-D block_mask"):
+        _check_blocks(q, k, 384, 384, torch.ones((1, 3, 2, 2), dtype=torch.bool))
+
+
+def test_no_cpu_fallback():
+    """CPU tensors are rejected: the product has no path that avoids the HIP kernels."""
+    import flex_block_attn_amd as fba
+
+    q = torch.zeros((1, 1, 128, 128), dtype=torch.bfloat16)
+    m = torch.ones((1, 1), dtype=torch.bool)
+    with pytest.raises(ValueError, match="GPU tensor"):
+        fba.flex_block_attn_func(q, q, q, 128, 128, m)
+    with pytest.raises(ValueError, match="GPU tensor"):
+        fba.compact_block_mask(m)
+    with pytest.raises(TypeError, match="bool"):
+        fba.compact_block_mask(m.to(torch.uint8))
+
+
+def test_tensor_contract():
+    from flex_block_attn_amd.interface import _check_qkv
+
+    class FakeCuda(torch.Tensor):
+        pass
+
+    good = torch.zeros((1, 2, 256, 128), dtype=torch.bfloat16)
+    with pytest.raises(ValueError, match="GPU tensor"):
+        _check_qkv(good, good, good)
+
+
+def test_mask_helpers():
+    from flex_block_attn_amd import masks
+
+    q = torch.zeros((1, 1, 1536, 128))
+    sel = masks.generate_selected_blocks(q, 384, 0.5, seed=3)
+    assert len(sel) == 4 * 2 and sel == masks.generate_selected_blocks(q, 384, 0.5, seed=3)
+    for i in range(4):
+        cols = [j for (r, j) in sel if r == i]
+        assert len(cols) == 2 and len(set(cols)) == 2
+    bm = masks.create_sparse_mask(q, 384, sel)
+    assert bm.shape == (4, 4) and bm.dtype == torch.bool and int(bm.sum()) == 8
+    dense = masks.create_torch_mask(q, 384, sel)
+    assert dense.shape == (1536, 1536) and torch.equal(dense[::384, ::384], bm)
+    assert torch.equal(dense, masks.expand_block_mask(bm, 384, 384))
+    swa = masks.generate_swa_selected_blocks(q, 384, 2)
+    assert set(swa) == {(i, j) for i in range(4) for j in range(4) if abs(i - j) < 2}
+    assert torch.equal(masks.create_sparse_mask(q, 384, swa), masks.swa_block_mask(4, 4, 2))
+
+    r = masks.random_block_mask(1, 3, 80, 80, 32, seed=0)
+    assert r.shape == (1, 3, 80, 80) and (r.sum(-1) == 32).all() and r.diagonal(dim1=-2, dim2=-1).all()
+    assert torch.equal(r, masks.random_block_mask(1, 3, 80, 80, 32, seed=0))
+    assert not torch.equal(r[0, 0], r[0, 1])
+
+    sta = masks.sta_3d_block_mask((5, 6, 10), (3, 3, 3), clamp=True)
+    assert sta.shape == (300, 300) and (sta.sum(-1) == 27).all() and sta.diagonal().all()
+    clipped = masks.sta_3d_block_mask((5, 6, 10), (3, 3, 3), clamp=False)
+    assert int(clipped.sum()) == 5824 and torch.equal(clipped, clipped.t())
+
+
+def test_block_lists_transposed_view():
+    from flex_block_attn_amd.interface import BlockLists
+
+    a, b, c, d = (torch.zeros(1) for _ in range(4))
+    t = BlockLists(a, b, c, d, 1, 3, 5).transposed()
+    assert t.q_cnt is c and t.q_idx is d and t.k_cnt is a and t.k_idx is b and (t.nQ, t.nK) == (5, 3)

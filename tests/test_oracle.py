@@ -1,0 +1,252 @@
+"""Pins the CPU oracle (oracle/attn_oracle.py, oracle/attn_ref.c) before anything is compared against it.
+
+The reference holds no golden vectors for this path; its one known-answer relation is "equals
+F.scaled_dot_product_attention on the dense expanded mask" (test/test_flex_block_attn.py:48-51, :139).  The checks
+below are chosen so that a plausible mistake fails one of them: three independent restatements must agree; special
+masks must reduce to textbook attention; tiny cases are brute-forced with Python loops; gradients are checked against
+fp64 finite differences and against identities that a dropped term or a transposed operand breaks.
+"""
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+TOL = 2e-5  # fp32 agreement between restatements
+
+
+def _mask(kind, nQ, nK, seed=0, B=1, H=1):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    if kind == "full":
+        return torch.ones((nQ, nK), dtype=torch.bool)
+    if kind == "diag":
+        return torch.eye(nQ, nK, dtype=torch.bool)
+    if kind == "rand2d":
+        m = torch.rand((nQ, nK), generator=g) < 0.5
+        m[torch.arange(nQ), (torch.arange(nQ) * nK) // nQ] = True
+        return m
+    if kind == "rand4d":
+        m = torch.rand((B, H, nQ, nK), generator=g) < 0.5
+        m[..., torch.arange(nQ), (torch.arange(nQ) * nK) // nQ] = True
+        return m
+    raise ValueError(kind)
+
+
+CASES = [
+    # B, Hq, Hkv, Sq, Skv, qbs, kbs, mask kind
+    (1, 2, 2, 64, 64, 16, 16, "rand2d"),
+    (2, 2, 2, 64, 96, 16, 32, "rand4d"),
+    (1, 4, 2, 32, 64, 16, 16, "rand4d"),  # grouped-query heads
+    (1, 1, 1, 48, 48, 16, 16, "full"),
+]
+
+
+@pytest.mark.parametrize("case", CASES)
+def test_three_restatements_agree(oracle, case):
+    B, Hq, Hkv, Sq, Skv, qbs, kbs, kind = case
+    q, k, v, do = oracle.seeded_qkv(B, Hq, Hkv, Sq, Skv, D=32, seed=1)
+    m = _mask(kind, Sq // qbs, Skv // kbs, seed=2, B=B, H=Hq)
+    o_e, lse_e = oracle.dense_attention_explicit(q, k, v, m, qbs, kbs)
+    o_s, dq_s, dk_s, dv_s = oracle.sdpa_dense(q, k, v, m, qbs, kbs, do)
+    o_c, lse_c = oracle.c_attention_forward(q, k, v, m, qbs, kbs)
+    assert oracle.error_metrics(o_e, o_s)[0] < TOL
+    assert oracle.error_metrics(o_c, o_s)[0] < TOL
+    assert oracle.error_metrics(lse_c, lse_e)[0] < TOL
+    g_e = oracle.dense_attention_backward_explicit(q, k, v, o_e, lse_e, do, m, qbs, kbs)
+    g_c = oracle.c_attention_backward(q, k, v, o_c, lse_c, do, m, qbs, kbs)
+    for ge, gc, gs in zip(g_e, g_c, (dq_s, dk_s, dv_s)):
+        assert ge.shape == gs.shape and gc.shape == gs.shape
+        assert oracle.error_metrics(ge, gs)[0] < 5 * TOL
+        assert oracle.error_metrics(gc, gs)[0] < 5 * TOL
+
+
+def test_full_mask_is_plain_attention(oracle):
+    q, k, v, _ = oracle.seeded_qkv(1, 2, 2, 64, 64, D=32, seed=3)
+    m = torch.ones((4, 4), dtype=torch.bool)
+    o, lse = oracle.c_attention_forward(q, k, v, m, 16, 16)
+    want = torch.nn.functional.scaled_dot_product_attention(q, k, v)
+    assert oracle.error_metrics(o, want)[0] < TOL
+    s = torch.matmul(q, k.transpose(-1, -2)) / math.sqrt(32)
+    assert oracle.error_metrics(lse, torch.logsumexp(s, -1))[0] < TOL
+
+
+def test_block_diagonal_is_independent_attentions(oracle):
+    q, k, v, _ = oracle.seeded_qkv(1, 1, 1, 64, 64, D=32, seed=4)
+    o, _ = oracle.c_attention_forward(q, k, v, torch.eye(4, dtype=torch.bool), 16, 16)
+    for i in range(4):
+        sl = slice(16 * i, 16 * i + 16)
+        want = torch.nn.functional.scaled_dot_product_attention(q[:, :, sl], k[:, :, sl], v[:, :, sl])
+        assert oracle.error_metrics(o[:, :, sl], want)[0] < TOL
+
+
+def test_rectangular_blocks_single_selection(oracle):
+    """q_block 16, kv_block 32: query block i attends key block (i // 2) only."""
+    q, k, v, _ = oracle.seeded_qkv(1, 1, 1, 64, 64, D=32, seed=5)
+    m = torch.zeros((4, 2), dtype=torch.bool)
+    for i in range(4):
+        m[i, i // 2] = True
+    o, _ = oracle.c_attention_forward(q, k, v, m, 16, 32)
+    for i in range(4):
+        qs, ks = slice(16 * i, 16 * i + 16), slice(32 * (i // 2), 32 * (i // 2) + 32)
+        want = torch.nn.functional.scaled_dot_product_attention(q[:, :, qs], k[:, :, ks], v[:, :, ks])
+        assert oracle.error_metrics(o[:, :, qs], want)[0] < TOL
+
+
+def test_brute_force_tiny(oracle):
+    """Pure-Python loops over every (query, key, channel) on a case small enough to read."""
+    B, H, S, D, bs = 1, 1, 8, 4, 2
+    q, k, v, do = oracle.seeded_qkv(B, H, H, S, S, D=D, seed=6)
+    m = _mask("rand2d", S // bs, S // bs, seed=7)
+    o_c, lse_c = oracle.c_attention_forward(q, k, v, m, bs, bs)
+    dq_c, dk_c, dv_c = oracle.c_attention_backward(q, k, v, o_c, lse_c, do, m, bs, bs)
+    Q, K, V, DO = (t[0, 0].double().tolist() for t in (q, k, v, do))
+    scale = 1.0 / math.sqrt(D)
+    O = [[0.0] * D for _ in range(S)]
+    P = [[0.0] * S for _ in range(S)]
+    for i in range(S):
+        sc = {j: scale * sum(Q[i][c] * K[j][c] for c in range(D)) for j in range(S) if m[i // bs, j // bs]}
+        mx = max(sc.values())
+        den = sum(math.exp(x - mx) for x in sc.values())
+        for j, x in sc.items():
+            P[i][j] = math.exp(x - mx) / den
+            for c in range(D):
+                O[i][c] += P[i][j] * V[j][c]
+        assert abs(lse_c[0, 0, i].item() - (mx + math.log(den))) < 1e-5
+    dQ = [[0.0] * D for _ in range(S)]
+    dK = [[0.0] * D for _ in range(S)]
+    dV = [[0.0] * D for _ in range(S)]
+    for i in range(S):
+        delta = sum(DO[i][c] * O[i][c] for c in range(D))
+        for j in range(S):
+            dp = sum(DO[i][c] * V[j][c] for c in range(D))
+            ds = P[i][j] * (dp - delta) * scale
+            for c in range(D):
+                dQ[i][c] += ds * K[j][c]
+                dK[j][c] += ds * Q[i][c]
+                dV[j][c] += P[i][j] * DO[i][c]
+    for got, want in ((o_c, O), (dq_c, dQ), (dk_c, dK), (dv_c, dV)):
+        assert (got[0, 0].double() - torch.tensor(want, dtype=torch.float64)).abs().max().item() < 1e-5
+
+
+def test_gradients_match_finite_differences_fp64(oracle):
+    B, Hq, Hkv, S, D, bs = 1, 2, 1, 8, 4, 4
+    q, k, v, do = (t.double() for t in oracle.seeded_qkv(B, Hq, Hkv, S, S, D=D, seed=8))
+    m = _mask("rand2d", S // bs, S // bs, seed=9)
+
+    def loss(q_, k_, v_):
+        o, _ = oracle.dense_attention_explicit(q_, k_, v_, m, bs, bs, dtype=torch.float64)
+        return (o * do).sum().item()
+
+    o, lse = oracle.dense_attention_explicit(q, k, v, m, bs, bs, dtype=torch.float64)
+    grads = oracle.dense_attention_backward_explicit(q, k, v, o, lse, do, m, bs, bs, dtype=torch.float64)
+    eps = 1e-6
+    for which, (x, g) in enumerate(zip((q, k, v), grads)):
+        flat = x.reshape(-1)
+        for pos in range(0, flat.numel(), 7):
+            xp, xm = flat.clone(), flat.clone()
+            xp[pos] += eps
+            xm[pos] -= eps
+            args_p = [q, k, v]
+            args_m = [q, k, v]
+            args_p[which] = xp.reshape(x.shape)
+            args_m[which] = xm.reshape(x.shape)
+            num = (loss(*args_p) - loss(*args_m)) / (2 * eps)
+            assert abs(num - g.reshape(-1)[pos].item()) < 1e-6, (which, pos)
+
+
+def test_gradient_identities(oracle):
+    """sum(q o dq) = sum(k o dk) per head (both equal sum_ij dS_ij S_ij); dK = dV = 0 for a key block nobody selects;
+    gradients are linear in dO."""
+    B, H, S, D, bs = 1, 2, 64, 32, 16
+    q, k, v, do = oracle.seeded_qkv(B, H, H, S, S, D=D, seed=10)
+    m = _mask("rand2d", 4, 4, seed=11)
+    m[:, 2] = False
+    o, lse = oracle.c_attention_forward(q, k, v, m, bs, bs)
+    dq, dk, dv = oracle.c_attention_backward(q, k, v, o, lse, do, m, bs, bs)
+    lhs, rhs = (q * dq).sum((-1, -2)), (k * dk).sum((-1, -2))
+    assert (lhs - rhs).abs().max().item() < 1e-3 * lhs.abs().max().item() + 1e-4
+    assert dk[:, :, 32:48].abs().max().item() == 0.0 and dv[:, :, 32:48].abs().max().item() == 0.0
+    dq2, dk2, dv2 = oracle.c_attention_backward(q, k, v, o, lse, 2 * do, m, bs, bs)
+    for a, b2 in ((dq, dq2), (dk, dk2), (dv, dv2)):
+        assert oracle.error_metrics(b2, 2 * a)[0] < 1e-5
+
+
+def test_key_block_permutation_invariance(oracle):
+    B, H, S, D, bs = 1, 1, 64, 32, 16
+    q, k, v, _ = oracle.seeded_qkv(B, H, H, S, S, D=D, seed=12)
+    m = _mask("rand2d", 4, 4, seed=13)
+    perm = torch.tensor([2, 0, 3, 1])
+    tok = (perm[:, None] * bs + torch.arange(bs)[None, :]).reshape(-1)
+    o1, lse1 = oracle.c_attention_forward(q, k, v, m, bs, bs)
+    o2, lse2 = oracle.c_attention_forward(q, k[:, :, tok], v[:, :, tok], m[:, perm], bs, bs)
+    assert oracle.error_metrics(o2, o1)[0] < TOL and oracle.error_metrics(lse2, lse1)[0] < TOL
+
+
+def test_empty_query_block(oracle):
+    """A query block that selects nothing: O = 0, LSE = -inf, dQ = 0 (the reference divides 0/0 there)."""
+    q, k, v, do = oracle.seeded_qkv(1, 1, 1, 32, 32, D=16, seed=14)
+    m = torch.tensor([[True, False], [False, False]])
+    o, lse = oracle.c_attention_forward(q, k, v, m, 16, 16)
+    assert o[0, 0, 16:].abs().max().item() == 0.0 and torch.isinf(lse[0, 0, 16:]).all() and (lse[0, 0, 16:] < 0).all()
+    o_e, lse_e = oracle.dense_attention_explicit(q, k, v, m, 16, 16)
+    assert torch.equal(torch.isinf(lse_e), torch.isinf(lse)) and oracle.error_metrics(o_e, o)[0] < TOL
+    dq, dk, dv = oracle.c_attention_backward(q, k, v, o, lse, do, m, 16, 16)
+    assert dq[0, 0, 16:].abs().max().item() == 0.0
+    assert torch.isfinite(dq).all() and torch.isfinite(dk).all() and torch.isfinite(dv).all()
+
+
+def test_mask_expansion(oracle):
+    m = _mask("rand2d", 3, 5, seed=15)
+    dense = oracle.expand_block_mask(m, 4, 2)
+    dense_c = oracle.c_expand_block_mask(m, 4, 2)
+    assert dense.shape == (12, 10) and torch.equal(dense, dense_c)
+    for i in range(12):
+        for j in range(10):
+            assert dense[i, j] == m[i // 4, j // 2]
+
+
+@pytest.mark.parametrize("shape", [(4, 4), (1, 1), (7, 9), (80, 80), (65, 129), (2, 3, 17, 70)])
+def test_compaction_lists(oracle, shape):
+    g = torch.Generator(device="cpu").manual_seed(sum(shape))
+    m = torch.rand(shape, generator=g) < 0.4
+    q_cnt, q_idx, k_cnt, k_idx = oracle.compact_lists(m)
+    c = oracle.c_compact_lists(m)
+    for a, b in zip((q_cnt, q_idx, k_cnt, k_idx), c):
+        assert a.dtype == np.int32 and np.array_equal(a, b)
+    m3 = m.reshape(-1, shape[-2], shape[-1])
+    assert q_cnt.sum() == k_cnt.sum() == int(m.sum())
+    for b in range(m3.shape[0]):
+        nz = torch.nonzero(m3[b])  # row-major: ascending (i, j)
+        for i in range(shape[-2]):
+            want = nz[nz[:, 0] == i][:, 1].numpy()
+            assert np.array_equal(q_idx[b, i, : q_cnt[b, i]], want)
+            assert (q_idx[b, i, q_cnt[b, i] :] == -1).all()
+        nzt = torch.nonzero(m3[b].t())
+        for j in range(shape[-1]):
+            want = nzt[nzt[:, 0] == j][:, 1].numpy()
+            assert np.array_equal(k_idx[b, j, : k_cnt[b, j]], want)
+            assert (k_idx[b, j, k_cnt[b, j] :] == -1).all()
+
+
+def test_golden_fixtures_match_oracle(oracle):
+    """The committed fixtures are what the oracle computes today (guards both against drift)."""
+    gdir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+    names = sorted(f for f in os.listdir(gdir) if f.endswith(".npz"))
+    assert len(names) >= 4
+    for name in names:
+        z = np.load(os.path.join(gdir, name))
+        q, k, v, do = (torch.from_numpy(z[n]).view(torch.bfloat16).float() for n in ("q", "k", "v", "do"))
+        m = torch.from_numpy(z["mask"])
+        qbs, kbs = int(z["q_block"]), int(z["kv_block"])
+        o_s, dq_s, dk_s, dv_s = oracle.sdpa_dense(q, k, v, m, qbs, kbs, do)
+        rows_ok = torch.isfinite(torch.from_numpy(z["lse"]))  # SDPA yields NaN on rows without keys
+        sel = rows_ok.unsqueeze(-1).expand_as(o_s)
+        assert (torch.from_numpy(z["o"])[sel] - o_s[sel]).abs().max().item() < 5 * TOL
+        if rows_ok.all():
+            scale = max(1.0, float(dq_s.abs().max()))
+            for n, want in (("dq", dq_s), ("dk", dk_s), ("dv", dv_s)):
+                assert (torch.from_numpy(z[n]) - want).abs().max().item() < 2e-4 * scale, (name, n)
+        lists = oracle.compact_lists(m)
+        for n, want in zip(("q_cnt", "q_idx", "k_cnt", "k_idx"), lists):
+            assert np.array_equal(z[n], want)
