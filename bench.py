@@ -26,6 +26,11 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 D = 128
 
+# HBM bytes per launch (2 x FETCH_SIZE + WRITE_SIZE KiB, the factors a plain copy of known size gives) from separate
+# rocprofv3 --pmc runs of this script; the counter summary is kept under profiles/.  Only the default workload has been
+# measured; other workloads report null.
+MEASURED_TRAFFIC = {"random": {"fwd": 5.73e9, "bwd_dkdv": 14.90e9, "bwd_dq": 5.90e9}}
+
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
@@ -107,6 +112,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="random")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 256 MiB device copy three times, as the known-size yardstick for rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU only: every box in this build has a single MI355X (use --gpus 1)")
@@ -170,7 +177,8 @@ def main():
     rooflines = {}
     for name, fl in kernel_flops.items():
         ach = fl / (kms[name]["mean_ms"] * 1e-3) * 1e-12
-        rooflines[name] = {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "ms": kms[name]["mean_ms"]}
+        rooflines[name] = {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_BF16_TFLOPS,
+                           "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get(name), "ms": kms[name]["mean_ms"]}
     dominant = max(kernel_flops, key=lambda n: kms[n]["mean_ms"])
     roofline = dict(rooflines[dominant])
     roofline["kernel"] = dominant
@@ -187,6 +195,14 @@ def main():
         "rooflines": rooflines,
         "mask_compaction": compaction,
     }
+
+    if args.calibrate_copy:
+        src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        log("calibration: 3 device copies of 268435456 bytes (read 256 MiB + write 256 MiB each)")
 
     cpu = None if args.no_cpu else cpu_baseline()
     out = {
