@@ -8,6 +8,8 @@ from .interface import (
     compact_block_mask,
     flex_block_attn_func,
     forward_with_lists,
+    lists_for,
+    tile_block_mask,
 )
 from . import masks
 
@@ -20,5 +22,7 @@ __all__ = [
     "compact_block_mask",
     "forward_with_lists",
     "backward_with_lists",
+    "lists_for",
+    "tile_block_mask",
     "masks",
 ]

@@ -76,23 +76,71 @@ int32_t fba_mask_compact(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32
   return e == hipSuccess ? FBA_OK : hip_fail(e, "mask_compact launch");
 }
 
-int32_t fba_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* q_cnt,
-                const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
-                int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+}  // extern "C"
+
+namespace {
+
+// Which list flavour a shape needs: block lists when both block sizes are multiples of the 128-row kernel tiles, tile
+// lists otherwise.  Tile lists need Sq and Skv to be multiples of 128.
+int check_lists(const Shape& s, bool tiled, const char* what) {
+  const bool aligned = s.q_block % 128 == 0 && s.k_block % 128 == 0;
+  if (!tiled && !aligned)
+    return fail(FBA_ERR_UNSUPPORTED, "%s: q_block (%d) and k_block (%d) are not both multiples of 128; build tile lists "
+                "with fba_tile_lists and call the _tiled entry point", what, s.q_block, s.k_block);
+  if (tiled && (s.Sq % 128 != 0 || s.Skv % 128 != 0))
+    return fail(FBA_ERR_UNSUPPORTED, "%s: tile lists need Sq (%d) and Skv (%d) to be multiples of 128", what, s.Sq, s.Skv);
+  return FBA_OK;
+}
+
+int fwd_impl(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* q_cnt, const int32_t* q_idx,
+             int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block,
+             int32_t k_block, void* hip_stream, bool tiled) {
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"o", o}})) return rc;
   if (!lse || !q_cnt || !q_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
-  if (q_block % 128 != 0)
-    return fail(FBA_ERR_UNSUPPORTED, "forward: q_block (%d) must be a multiple of 128 in this build", q_block);
+  if (int rc = check_lists(s, tiled, "forward")) return rc;
   fba::FwdParams p{};
   p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.o = (__bf16*)o; p.lse = lse;
   p.q_cnt = q_cnt; p.q_idx = q_idx; p.mask_bh = mask_bh;
   p.B = B; p.Hq = Hq; p.Hkv = Hkv; p.Sq = Sq; p.Skv = Skv; p.nQ = Sq / q_block; p.nK = Skv / k_block;
   p.q_block = q_block; p.k_block = k_block;
   p.scale_log2e = 1.4426950408889634f / 11.313708498984761f;
+  p.tiled = tiled ? 1 : 0;
   hipError_t e = fba::launch_fwd(p, (hipStream_t)hip_stream);
   return e == hipSuccess ? FBA_OK : hip_fail(e, "forward launch");
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t fba_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* q_cnt,
+                const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
+                int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+  return fwd_impl(q, k, v, o, lse, q_cnt, q_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream, false);
+}
+
+int32_t fba_fwd_tiled(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* qt_cnt,
+                      const int32_t* qt_ent, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
+                      int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+  return fwd_impl(q, k, v, o, lse, qt_cnt, qt_ent, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream, true);
+}
+
+int32_t fba_tile_lists(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32_t nK, int32_t q_block, int32_t k_block,
+                       int32_t* qt_cnt, int32_t* qt_ent, int32_t* kt_cnt, int32_t* kt_ent, void* hip_stream) {
+  if (mask_bh <= 0 || nQ <= 0 || nK <= 0)
+    return fail(FBA_ERR_INVALID, "mask_bh, nQ, nK must be positive (got %lld %d %d)", (long long)mask_bh, nQ, nK);
+  if (q_block <= 0 || q_block % 16 != 0) return fail(FBA_ERR_INVALID, "q_block (%d) must be a positive multiple of 16", q_block);
+  if (k_block <= 0 || k_block % 64 != 0) return fail(FBA_ERR_INVALID, "k_block (%d) must be a positive multiple of 64", k_block);
+  const int64_t Sq = (int64_t)nQ * q_block, Skv = (int64_t)nK * k_block;
+  if (Sq % 128 != 0 || Skv % 128 != 0)
+    return fail(FBA_ERR_UNSUPPORTED, "tile lists need Sq (%lld) and Skv (%lld) to be multiples of 128", (long long)Sq, (long long)Skv);
+  if (Sq / 32 >= (1 << 23) || nK >= (1 << 23)) return fail(FBA_ERR_INVALID, "sequence too long for 24-bit list entries");
+  if (!mask || !qt_cnt || !qt_ent || !kt_cnt || !kt_ent) return fail(FBA_ERR_INVALID, "null pointer argument");
+  hipError_t e = fba::launch_tile_lists(mask, mask_bh, nQ, nK, q_block, k_block, (int)(Sq / 128), (int)(Skv / 128), (int)(Sq / 32),
+                                        qt_cnt, qt_ent, kt_cnt, kt_ent, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "tile_lists launch");
 }
 
 static int fill_bwd(fba::BwdParams& p, const Shape& s) {
@@ -114,56 +162,81 @@ int32_t fba_bwd_stats(const void* o, const void* d_o, const float* lse, float* s
   return e == hipSuccess ? FBA_OK : hip_fail(e, "stats launch");
 }
 
-int32_t fba_bwd_dq(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dq,
+static int dq_impl(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dq,
                    const int32_t* q_cnt, const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
-                   int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+                   int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream, bool tiled) {
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"d_o", d_o}, {"dq", dq}})) return rc;
   if (!stats || !q_cnt || !q_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
-  if (q_block % 128 != 0)
-    return fail(FBA_ERR_UNSUPPORTED, "dq: q_block (%d) must be a multiple of 128 in this build", q_block);
+  if (int rc = check_lists(s, tiled, "dq")) return rc;
   fba::BwdParams p{};
   fill_bwd(p, s);
+  p.tiled = tiled ? 1 : 0;
   p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.d_o = (const __bf16*)d_o;
   p.stats = stats; p.dq = (__bf16*)dq; p.q_cnt = q_cnt; p.q_idx = q_idx;
   hipError_t e = fba::launch_bwd_dq(p, (hipStream_t)hip_stream);
   return e == hipSuccess ? FBA_OK : hip_fail(e, "dq launch");
 }
 
-int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,
+static int dkdv_impl(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,
                      const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
-                     int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+                     int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream, bool tiled) {
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"d_o", d_o}, {"dk", dk}, {"dv", dv}})) return rc;
   if (!stats || !k_cnt || !k_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
-  if (k_block % 128 != 0)
-    return fail(FBA_ERR_UNSUPPORTED, "dkdv: k_block (%d) must be a multiple of 128 in this build", k_block);
-  if (q_block % 128 != 0)
-    return fail(FBA_ERR_UNSUPPORTED, "dkdv: q_block (%d) must be a multiple of 128 in this build", q_block);
+  if (int rc = check_lists(s, tiled, "dkdv")) return rc;
   if ((int64_t)B * Hq * Sq >= (1LL << 30)) return fail(FBA_ERR_INVALID, "B*Hq*Sq must be below 2^30");
   fba::BwdParams p{};
   fill_bwd(p, s);
+  p.tiled = tiled ? 1 : 0;
   p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.d_o = (const __bf16*)d_o;
   p.stats = stats; p.dk = (__bf16*)dk; p.dv = (__bf16*)dv; p.k_cnt = k_cnt; p.k_idx = k_idx;
   hipError_t e = fba::launch_bwd_dkdv(p, (hipStream_t)hip_stream);
   return e == hipSuccess ? FBA_OK : hip_fail(e, "dkdv launch");
 }
 
+static int bwd_impl(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                    float* stats, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
+                    const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
+                    int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream, bool tiled) {
+  const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
+  if (int rc = check_shape(s)) return rc;
+  if (int rc = check_lists(s, tiled, "backward")) return rc;
+  if (int rc = fba_bwd_stats(o, d_o, lse, stats, (int64_t)B * Hq * Sq, head_dim, hip_stream)) return rc;
+  if (int rc = dkdv_impl(q, k, v, d_o, stats, dk, dv, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block,
+                         hip_stream, tiled))
+    return rc;
+  return dq_impl(q, k, v, d_o, stats, dq, q_cnt, q_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream, tiled);
+}
+
+int32_t fba_bwd_dq(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dq,
+                   const int32_t* q_cnt, const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
+                   int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+  return dq_impl(q, k, v, d_o, stats, dq, q_cnt, q_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream, false);
+}
+
+int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,
+                     const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
+                     int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+  return dkdv_impl(q, k, v, d_o, stats, dk, dv, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream, false);
+}
+
 int32_t fba_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                 float* stats, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
                 const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
                 int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
-  const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
-  if (int rc = check_shape(s)) return rc;
-  if (q_block % 128 != 0 || k_block % 128 != 0)
-    return fail(FBA_ERR_UNSUPPORTED, "backward: q_block (%d) and k_block (%d) must be multiples of 128 in this build", q_block, k_block);
-  if (int rc = fba_bwd_stats(o, d_o, lse, stats, (int64_t)B * Hq * Sq, head_dim, hip_stream)) return rc;
-  if (int rc = fba_bwd_dkdv(q, k, v, d_o, stats, dk, dv, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block,
-                            hip_stream))
-    return rc;
-  return fba_bwd_dq(q, k, v, d_o, stats, dq, q_cnt, q_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream);
+  return bwd_impl(q, k, v, o, d_o, lse, stats, dq, dk, dv, q_cnt, q_idx, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim,
+                  q_block, k_block, hip_stream, false);
+}
+
+int32_t fba_bwd_tiled(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                      float* stats, void* dq, void* dk, void* dv, const int32_t* qt_cnt, const int32_t* qt_ent,
+                      const int32_t* kt_cnt, const int32_t* kt_ent, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
+                      int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+  return bwd_impl(q, k, v, o, d_o, lse, stats, dq, dk, dv, qt_cnt, qt_ent, kt_cnt, kt_ent, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim,
+                  q_block, k_block, hip_stream, true);
 }
 
 }  // extern "C"

@@ -31,8 +31,16 @@ constexpr int kRing = 4;
 template <int N>
 using IC = std::integral_constant<int, N>;
 
+// ring slot of a step: a compile-time constant in the unrolled loop, a run-time value in the rolled one
+template <int N>
+FBA_DEVICE constexpr int ring_of(IC<N>) { return N; }
+FBA_DEVICE int ring_of(int r) { return r; }
+
 }  // namespace
 
+// kTiled = false: q_block and k_block are multiples of 128; list entries are query blocks, expanded to q_block/32 slabs.
+// kTiled = true: tile lists; list entries are 32-row query slabs with a predicate per (wave, 16-row half-slab).
+template <bool kTiled>
 __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];  // ring [4] of (Q slab | dO slab | lse2 | delta)
   constexpr int TK = 128;
@@ -57,10 +65,11 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
     vreg[ks] = *reinterpret_cast<const bf16x8*>(p.v + (krow0 + l32) * kHeadDim + 16 * ks + 8 * h);
   }
 
-  const int nsub = p.q_block / kSlab;
+  const int nsub = kTiled ? 1 : p.q_block / kSlab;
+  const int row_len = kTiled ? p.Sq / kSlab : p.nQ;  // entries per list row
   auto list_row = [&](int g) -> int64_t {
     const int64_t bh = (int64_t)b * p.Hq + hkv * group + g;
-    return (p.mask_bh == 1 ? 0 : bh) * p.nK + kblk;
+    return (p.mask_bh == 1 ? 0 : bh) * (kTiled ? tiles_per_head : p.nK) + (kTiled ? kt : kblk);
   };
   const ConstIdx k_cnt = const_idx(p.k_cnt);
   int nsteps = 0;
@@ -98,11 +107,11 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
       if (++g_cur >= group) return;
       const int64_t lr = list_row(g_cur);
       cnt_cur = k_cnt[lr];
-      idx_cur = const_idx(p.k_idx + lr * p.nQ);
+      idx_cur = const_idx(p.k_idx + lr * row_len);
       head_row0 = ((int64_t)b * p.Hq + hkv * group + g_cur) * p.Sq;
       e_cur = 0;
     }
-    row_next = head_row0 + (int64_t)idx_cur[e_cur] * p.q_block;
+    row_next = head_row0 + (kTiled ? (int64_t)(idx_cur[e_cur] >> 8) * kSlab : (int64_t)idx_cur[e_cur] * p.q_block);
     rem = nsub;
   };
   auto copy_next = [&](int ring) {
@@ -136,14 +145,35 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
     for (int ks = 0; ks < 8; ++ks) { pin(kreg[ks]); pin(vreg[ks]); }
     f32x16 s_cur, dp_cur;
     scores(smem, s_cur, dp_cur);
+    // tile lists: predicate bits of the slab being computed, from a second walk over the same lists
+    int g_cmp = -1, e_cmp = 0, cnt_cmp = 0, bits_cmp = 0;
+    ConstIdx idx_cmp = nullptr;
+    auto next_bits = [&]() {
+      ++e_cmp;
+      while (e_cmp >= cnt_cmp) {
+        if (++g_cmp >= group) { bits_cmp = 0; return; }
+        const int64_t lr = list_row(g_cmp);
+        cnt_cmp = k_cnt[lr];
+        idx_cmp = const_idx(p.k_idx + lr * row_len);
+        e_cmp = 0;
+      }
+      bits_cmp = idx_cmp[e_cmp] & 255;
+    };
+    if constexpr (kTiled) {
+      e_cmp = -1;
+      next_bits();
+    }
 
     // step t (t % 4 == R): P_t, dS_t from (S_t, dP_t) | S_{t+1}, dP_{t+1} from slab t+1 | dV += dO_t^T P_t, dK += Q_t^T dS_t
     auto step = [&](auto ring_c, int t) {
-      constexpr int R = decltype(ring_c)::value;
+      const int R = ring_of(ring_c);
       const char* stage = smem + R * kStageBytes;
       f32x16 s_nxt, dp_nxt;
       scores(smem + ((R + 1) & 3) * kStageBytes, s_nxt, dp_nxt);  // past the last slab: stale data, unused
       const float* st_lds = reinterpret_cast<const float*>(stage + 2 * kSlabBytes);
+      // does this wave's key block select the first / second 16 query rows of the slab?
+      const bool on0 = !kTiled || ((bits_cmp >> (2 * wave)) & 1) != 0;
+      const bool on1 = !kTiled || ((bits_cmp >> (2 * wave + 1)) & 1) != 0;
       // accumulator element 4g + e of half-wave h is query row 8g + 4h + e of the slab
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -151,7 +181,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
         const f32x4 d4 = *reinterpret_cast<const f32x4*>(st_lds + kSlab + 8 * g + 4 * h);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const float pv = fast_exp2(__builtin_fmaf(s_cur[4 * g + e], c, -l4[e]));
+          float pv = fast_exp2(__builtin_fmaf(s_cur[4 * g + e], c, -l4[e]));
+          if constexpr (kTiled) pv = (g < 2 ? on0 : on1) ? pv : 0.f;  // a select: inf or NaN of a masked row is discarded
           s_cur[4 * g + e] = pv;
           dp_cur[4 * g + e] = pv * (dp_cur[4 * g + e] - d4[e]);
         }
@@ -176,16 +207,21 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
         }
       s_cur = s_nxt;
       dp_cur = dp_nxt;
+      if constexpr (kTiled) next_bits();
       // slab t+2 must have landed (first read in step t+1); the five copies of slab t+3 may still fly
       if (t + 3 < nsteps) wait_vmem<5>(); else wait_vmem<0>();
       __syncthreads();
       if (t + 4 < nsteps) copy_next(R);
     };
-    for (int t = 0; t < nsteps; t += 4) {  // nsteps is a multiple of 4
-      step(IC<0>{}, t);
-      step(IC<1>{}, t + 1);
-      step(IC<2>{}, t + 2);
-      step(IC<3>{}, t + 3);
+    if constexpr (kTiled) {
+      for (int t = 0; t < nsteps; ++t) step(t & 3, t);  // any step count; ring slot computed at run time
+    } else {
+      for (int t = 0; t < nsteps; t += 4) {  // nsteps is a multiple of 4
+        step(IC<0>{}, t);
+        step(IC<1>{}, t + 1);
+        step(IC<2>{}, t + 2);
+        step(IC<3>{}, t + 3);
+      }
     }
   }
 
@@ -207,9 +243,13 @@ hipError_t launch_bwd_dkdv(BwdParams p, hipStream_t stream) {
   constexpr int kSmem = kRing * kStageBytes;
   p.num_items = p.B * p.Hkv * (p.Skv / 128);
   p.items_per_xcd = (p.num_items + kNumXcd - 1) / kNumXcd;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dkdv_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
+  const void* fn = p.tiled ? reinterpret_cast<const void*>(&dkdv_kernel<true>) : reinterpret_cast<const void*>(&dkdv_kernel<false>);
+  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(dkdv_kernel, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
+  if (p.tiled)
+    hipLaunchKernelGGL(dkdv_kernel<true>, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
+  else
+    hipLaunchKernelGGL(dkdv_kernel<false>, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
   return hipGetLastError();
 }
 

@@ -43,6 +43,8 @@ using IC = std::integral_constant<int, N>;
 #else
 #define FBA_DQ_OCCUPANCY , amdgpu_waves_per_eu(2, 2)
 #endif
+// kTiled: see the forward kernel (tile lists with a predicate per 16-row group instead of block lists).
+template <bool kTiled>
 __global__ __attribute__((amdgpu_flat_work_group_size(256, 256) FBA_DQ_OCCUPANCY)) void dq_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];  // ring [4] of (K slab | V slab)
   constexpr int TQ = 128;
@@ -61,10 +63,11 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256) FBA_DQ_OCCUPANCY
   const char* kp = reinterpret_cast<const char*>(p.k + ((int64_t)(b * p.Hkv + hkv) * p.Skv) * kHeadDim);
   const char* vp = reinterpret_cast<const char*>(p.v + ((int64_t)(b * p.Hkv + hkv) * p.Skv) * kHeadDim);
 
-  const int qblk = (qt * TQ) / p.q_block;
-  const int64_t mrow = (p.mask_bh == 1 ? 0 : (int64_t)bh) * p.nQ + qblk;
+  const int64_t mrow = (p.mask_bh == 1 ? 0 : (int64_t)bh) * (kTiled ? tiles_per_head : p.nQ) + (kTiled ? qt : (qt * TQ) / p.q_block);
   const int cnt = p.q_cnt[mrow];
   const ConstIdx idx = const_idx(p.q_idx + mrow * p.nK);
+  auto key_block = [&](int e) -> int { return kTiled ? idx[e] >> 8 : idx[e]; };
+  const int group_bit = 1 << (2 * wave + (l32 >> 4));  // this lane's 16-row group in a tile-list entry
   const int nsub = p.k_block / kSlab;
   const int nsteps = cnt * nsub;
 
@@ -97,8 +100,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256) FBA_DQ_OCCUPANCY
   // slab source offsets in list order; the list entry of the following key block is read one block ahead
   const int64_t block_bytes = (int64_t)p.k_block * kRowBytes;
   int e_next = 1, rem = nsub;
-  int64_t src_off = cnt > 0 ? idx[0] * block_bytes : 0;
-  int blk_next = cnt > 1 ? idx[1] : 0;
+  int64_t src_off = cnt > 0 ? key_block(0) * block_bytes : 0;
+  int blk_next = cnt > 1 ? key_block(1) : 0;
   auto copy_next = [&](int ring) {
     dma.copy(ring_dst + ring * kPairBytes, kp + src_off);
     dma.copy(ring_dst + ring * kPairBytes + kSlabBytes, vp + src_off);
@@ -106,7 +109,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256) FBA_DQ_OCCUPANCY
       rem = nsub;
       src_off = blk_next * block_bytes;
       ++e_next;
-      blk_next = e_next < cnt ? idx[e_next] : 0;
+      blk_next = e_next < cnt ? key_block(e_next) : 0;
     } else {
       src_off += kSlabBytes;
     }
@@ -136,9 +139,13 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256) FBA_DQ_OCCUPANCY
     scores(smem, s_cur, dp_cur);
 #endif
 
+    int e_cmp = 0, rem_cmp = nsub;  // list entry of the slab being computed (tile lists: its predicate bits)
+    int bits_cmp = kTiled ? idx[0] & 255 : 255;
+
     // step t (t % 4 == R): dS_t from (S_t, dP_t) | S_{t+1}, dP_{t+1} from slab t+1 | dQ += K_t^T dS_t
     auto step = [&](auto ring_c, int t) {
       constexpr int R = decltype(ring_c)::value;
+      const bool active = !kTiled || (bits_cmp & group_bit) != 0;
 #if FBA_DQ_PIPELINED
       f32x16 s_nxt, dp_nxt;
       scores(smem + ((R + 1) & 3) * kPairBytes, s_nxt, dp_nxt);  // past the last slab: stale data, unused
@@ -148,7 +155,18 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256) FBA_DQ_OCCUPANCY
 #endif
       bf16x8 dsk[2];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) s_cur[r] = fast_exp2(__builtin_fmaf(s_cur[r], c, -lse2)) * (dp_cur[r] - dlt);
+      for (int r = 0; r < 16; ++r) {
+        float pv = fast_exp2(__builtin_fmaf(s_cur[r], c, -lse2));
+        if constexpr (kTiled) pv = active ? pv : 0.f;  // a select, so that inf or NaN of a masked row is discarded
+        s_cur[r] = pv * (dp_cur[r] - dlt);
+      }
+      if constexpr (kTiled) {
+        if (--rem_cmp == 0) {
+          rem_cmp = nsub;
+          ++e_cmp;
+          bits_cmp = e_cmp < cnt ? idx[e_cmp] & 255 : 0;
+        }
+      }
 #pragma unroll
       for (int j = 0; j < 2; ++j)
         dsk[j] = pack8(s_cur[8 * j + 0], s_cur[8 * j + 1], s_cur[8 * j + 2], s_cur[8 * j + 3], s_cur[8 * j + 4],
@@ -195,9 +213,13 @@ hipError_t launch_bwd_dq(BwdParams p, hipStream_t stream) {
   constexpr int kSmem = kRing * kPairBytes;
   p.num_items = p.B * p.Hq * (p.Sq / 128);
   p.items_per_xcd = (p.num_items + kNumXcd - 1) / kNumXcd;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
+  const void* fn = p.tiled ? reinterpret_cast<const void*>(&dq_kernel<true>) : reinterpret_cast<const void*>(&dq_kernel<false>);
+  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(dq_kernel, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
+  if (p.tiled)
+    hipLaunchKernelGGL(dq_kernel<true>, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
+  else
+    hipLaunchKernelGGL(dq_kernel<false>, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
   return hipGetLastError();
 }
 

@@ -81,11 +81,12 @@ FBA_DEVICE void pv_half(FwdState& st, const char* v_half, const bf16x8 (&pk)[2])
 
 // Raise the softmax reference if some row of the wave would otherwise see exponents above kLazy.  Until then
 // P = exp2(c (S - m)) may exceed 1, which fp32 sums and bf16 P both carry.
-FBA_DEVICE void softmax_reference(FwdState& st, const f32x16& s) {
+// `active` is false for a query row whose own mask block does not select the current key block (tile lists only).
+FBA_DEVICE void softmax_reference(FwdState& st, const f32x16& s, bool active) {
   float mx = s[0];
 #pragma unroll
   for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[r]);
-  mx = max_halves(mx);
+  mx = max_halves(active ? mx : -INFINITY);
   if (__builtin_amdgcn_ballot_w64((mx - st.m_run) * st.c > kLazy) != 0) {
     const float m_new = fmaxf(st.m_run, mx);
     const float alpha = fast_exp2((st.m_run - m_new) * st.c);
@@ -100,16 +101,21 @@ FBA_DEVICE void softmax_reference(FwdState& st, const f32x16& s) {
 }
 
 // P^T = exp2(c S^T - c m), packed to bf16 as the B operand of the two 16-key MFMA steps.
-FBA_DEVICE void softmax_exp(FwdState& st, f32x16& s, bf16x8 (&pk)[2]) {
+template <bool kTiled>
+FBA_DEVICE void softmax_exp(FwdState& st, f32x16& s, bf16x8 (&pk)[2], bool active) {
   const float mc = st.m_run * st.c;
 #if FBA_FWD_MFMA_ROWSUM
 #pragma unroll
-  for (int r = 0; r < 16; ++r) s[r] = fast_exp2(__builtin_fmaf(s[r], st.c, -mc));
+  for (int r = 0; r < 16; ++r) {
+    s[r] = fast_exp2(__builtin_fmaf(s[r], st.c, -mc));
+    if constexpr (kTiled) s[r] = active ? s[r] : 0.f;
+  }
 #else
   float rs = 0.f;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     s[r] = fast_exp2(__builtin_fmaf(s[r], st.c, -mc));
+    if constexpr (kTiled) s[r] = active ? s[r] : 0.f;
     rs += s[r];
   }
   st.acc_l[0] += rs;  // partial sum of this half-wave's keys
@@ -121,6 +127,9 @@ FBA_DEVICE void softmax_exp(FwdState& st, f32x16& s, bf16x8 (&pk)[2]) {
 
 }  // namespace
 
+// kTiled = false: q_block is a multiple of 128, the list of a work-group is the block list of its query block.
+// kTiled = true: tile lists with a predicate per 16-row group (any q_block that is a multiple of 16).
+template <bool kTiled>
 __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_per_eu(2, 2))) void fwd_kernel(const FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];  // K ring [4][8 KiB] | V ring [4][8 KiB]
   constexpr int TQ = 128;
@@ -140,10 +149,12 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   const char* kp = reinterpret_cast<const char*>(p.k + ((int64_t)(b * p.Hkv + hkv) * p.Skv) * kHeadDim);
   const char* vp = reinterpret_cast<const char*>(p.v + ((int64_t)(b * p.Hkv + hkv) * p.Skv) * kHeadDim);
 
-  const int qblk = (qt * TQ) / p.q_block;
-  const int64_t mrow = (p.mask_bh == 1 ? 0 : (int64_t)bh) * p.nQ + qblk;
+  const int64_t mrow = (p.mask_bh == 1 ? 0 : (int64_t)bh) * (kTiled ? tiles_per_head : p.nQ) + (kTiled ? qt : (qt * TQ) / p.q_block);
   const int cnt = p.q_cnt[mrow];
   const ConstIdx idx = const_idx(p.q_idx + mrow * p.nK);
+  auto key_block = [&](int e) -> int { return kTiled ? idx[e] >> 8 : idx[e]; };
+  // predicate bit of this lane's 16-row group in a tile-list entry
+  const int group_bit = 1 << (2 * wave + (l32 >> 4));
   const int nsub = p.k_block / kSlab;
   const int nsteps = cnt * nsub;
 
@@ -154,7 +165,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   st.rm.init(lane);
   st.tr.init(lane);
   st.c = p.scale_log2e;
-  st.m_run = -INFINITY;
+  st.m_run = kTiled ? -1e30f : -INFINITY;  // finite where whole slabs can be masked out, so that exp2 never sees inf - inf
 #pragma unroll
   for (int t = 0; t < 8; ++t) st.ones[t] = (__bf16)1.f;
 #pragma unroll
@@ -175,15 +186,15 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   // the scalar load is off the critical path.  V requests trail K requests by two slabs and reuse their offsets.
   const int64_t block_bytes = (int64_t)p.k_block * kRowBytes;
   int e_next = 1, rem = nsub;
-  int64_t src_off = cnt > 0 ? idx[0] * block_bytes : 0;
-  int blk_next = cnt > 1 ? idx[1] : 0;
+  int64_t src_off = cnt > 0 ? key_block(0) * block_bytes : 0;
+  int blk_next = cnt > 1 ? key_block(1) : 0;
   auto next_off = [&]() -> int64_t {
     const int64_t off = src_off;
     if (--rem == 0) {
       rem = nsub;
       src_off = blk_next * block_bytes;
       ++e_next;
-      blk_next = e_next < cnt ? idx[e_next] : 0;
+      blk_next = e_next < cnt ? key_block(e_next) : 0;
     } else {
       src_off += kSlabBytes;
     }
@@ -217,6 +228,9 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     int64_t hist0 = off[4], hist1 = off[3];  // offsets of the two youngest K requests
 
     bf16x8 p_prev[2];
+    // predicate of the slab whose softmax is next (tile lists): all 16-row groups share the entry, each lane tests its bit
+    int e_cmp = 0, rem_cmp = nsub;
+    int bits_cmp = kTiled ? idx[0] & 255 : 255;
 
     // step t (t % 4 == R): O += P_{t-1} V_{t-1} | softmax(S_t) | S_{t+1} = K_{t+1} Q^T
     auto step = [&](auto ring_c, auto first_c, int t) {
@@ -224,9 +238,17 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
       constexpr bool kFirst = decltype(first_c)::value;
       // P_{t-1} was formed against the reference m of step t-1, so it must reach O before step t may raise m
       if constexpr (!kFirst) pv_half(st, v_lds + ((R + 3) & 3) * kSlabBytes, p_prev);
-      softmax_reference(st, s_cur);
+      const bool active = !kTiled || (bits_cmp & group_bit) != 0;
+      softmax_reference(st, s_cur, active);
       const f32x16 s_nxt = qk_half(st, k_lds + ((R + 1) & 3) * kSlabBytes);  // past the last slab: stale data, unused
-      softmax_exp(st, s_cur, p_prev);  // p_prev := P_t
+      softmax_exp<kTiled>(st, s_cur, p_prev, active);  // p_prev := P_t
+      if constexpr (kTiled) {
+        if (--rem_cmp == 0) {
+          rem_cmp = nsub;
+          ++e_cmp;
+          bits_cmp = e_cmp < cnt ? idx[e_cmp] & 255 : 0;
+        }
+      }
       // P_t is only consumed after the barrier; without the pins its arithmetic sinks there, away from the MFMAs it is
       // meant to overlap with
       pin(p_prev[0]);
@@ -279,9 +301,13 @@ hipError_t launch_fwd(FwdParams p, hipStream_t stream) {
   constexpr int kSmem = 2 * kRing * kSlabBytes;
   p.num_items = p.B * p.Hq * (p.Sq / 128);
   p.items_per_xcd = (p.num_items + kNumXcd - 1) / kNumXcd;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&fwd_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
+  const void* fn = p.tiled ? reinterpret_cast<const void*>(&fwd_kernel<true>) : reinterpret_cast<const void*>(&fwd_kernel<false>);
+  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(fwd_kernel, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
+  if (p.tiled)
+    hipLaunchKernelGGL(fwd_kernel<true>, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
+  else
+    hipLaunchKernelGGL(fwd_kernel<false>, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
   return hipGetLastError();
 }
 

@@ -23,6 +23,9 @@ struct FwdParams {
   int B, Hq, Hkv, Sq, Skv, nQ, nK, q_block, k_block;
   float scale_log2e;  // log2(e) / sqrt(head_dim)
   int num_items, items_per_xcd;
+  // tiled = 1: q_cnt / q_idx are tile lists (qt_cnt [mask_bh, Sq/128], qt_ent [mask_bh, Sq/128, nK], see
+  // tile_lists_kernel) instead of block lists
+  int tiled;
 };
 
 struct BwdParams {
@@ -43,10 +46,16 @@ struct BwdParams {
   float scale;        // 1 / sqrt(head_dim)
   float scale_log2e;  // log2(e) / sqrt(head_dim)
   int num_items, items_per_xcd;
+  // tiled = 1: q_cnt / q_idx are qt_cnt / qt_ent and k_cnt / k_idx are kt_cnt [mask_bh, Skv/128] /
+  // kt_ent [mask_bh, Skv/128, Sq/32] (see tile_lists_kernel)
+  int tiled;
 };
 
 hipError_t launch_mask_compact(const uint8_t* mask, int64_t mask_bh, int nQ, int nK, int32_t* q_cnt, int32_t* q_idx,
                                int32_t* k_cnt, int32_t* k_idx, hipStream_t stream);
+hipError_t launch_tile_lists(const uint8_t* mask, int64_t mask_bh, int nQ, int nK, int q_block, int k_block, int n_qt,
+                             int n_kt, int n_qs, int32_t* qt_cnt, int32_t* qt_ent, int32_t* kt_cnt, int32_t* kt_ent,
+                             hipStream_t stream);
 hipError_t launch_fwd(FwdParams p, hipStream_t stream);
 hipError_t launch_bwd_stats(const __bf16* o, const __bf16* d_o, const float* lse, float* stats, int64_t rows, hipStream_t stream);
 hipError_t launch_bwd_dq(BwdParams p, hipStream_t stream);

@@ -54,6 +54,68 @@ hipError_t launch_mask_compact(const uint8_t* mask, int64_t mask_bh, int nQ, int
   return hipGetLastError();
 }
 
+// Tile lists for block sizes that do not align with the kernels' 128-row tiles (q_block or k_block not a multiple of
+// 128).  The attention kernels then work on 128-row tiles that straddle mask blocks, so every list entry carries a
+// predicate per 16-row group (query side) or per (wave, 16-row half-slab) pair (key side):
+//   qt_ent[m, T, 0..qt_cnt) = (J << 8) | bits, ascending J: key block J is selected by at least one of the eight 16-row
+//       groups of query tile T; bit g is mask[m, (128 T + 16 g) / q_block, J].                       (forward, dQ)
+//   kt_ent[m, U, 0..kt_cnt) = (s << 8) | bits, ascending s: 32-row query slab s touches key tile U; bit 2w + f is
+//       mask[m, (32 s + 16 f) / q_block, (128 U + 32 w) / k_block], w = wave (32 keys), f = half of the slab.  (dK/dV)
+// One wave per output row, same ballot / prefix-popcount compaction as above; unused entries are -1.
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void tile_lists_kernel(
+    const uint8_t* __restrict__ mask, int64_t mask_bh, int nQ, int nK, int q_block, int k_block, int n_qt, int n_kt,
+    int n_qs, int32_t* __restrict__ qt_cnt, int32_t* __restrict__ qt_ent, int32_t* __restrict__ kt_cnt,
+    int32_t* __restrict__ kt_ent) {
+  const int lane = threadIdx.x & 63;
+  const int64_t w = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int64_t n_qrows = mask_bh * n_qt, n_krows = mask_bh * n_kt;
+  if (w >= n_qrows + n_krows) return;
+  const bool q_pass = w < n_qrows;
+  const int64_t r = q_pass ? w : w - n_qrows;
+  const int per = q_pass ? n_qt : n_kt;
+  const int64_t m = r / per;
+  const int tile = (int)(r - m * per);
+  const uint8_t* base = mask + m * (int64_t)nQ * nK;
+  const int len = q_pass ? nK : n_qs;
+  int32_t* out = (q_pass ? qt_ent : kt_ent) + r * (int64_t)len;
+
+  int cnt = 0;
+  for (int t0 = 0; t0 < len; t0 += 64) {
+    const int t = t0 + lane;
+    int bits = 0;
+    if (t < len) {
+      if (q_pass) {
+#pragma unroll
+        for (int g = 0; g < 8; ++g) bits |= (base[(int64_t)((128 * tile + 16 * g) / q_block) * nK + t] != 0) << g;
+      } else {
+#pragma unroll
+        for (int wv = 0; wv < 4; ++wv)
+#pragma unroll
+          for (int f = 0; f < 2; ++f)
+            bits |= (base[(int64_t)((32 * t + 16 * f) / q_block) * nK + (128 * tile + 32 * wv) / k_block] != 0) << (2 * wv + f);
+      }
+    }
+    const bool on = bits != 0;
+    const unsigned long long bal = __ballot(on);
+    if (on) out[cnt + __popcll(bal & ((1ull << lane) - 1ull))] = (t << 8) | bits;
+    cnt += __popcll(bal);
+  }
+  for (int t = cnt + lane; t < len; t += 64) out[t] = -1;
+  if (lane == 0) (q_pass ? qt_cnt : kt_cnt)[r] = cnt;
+}
+
+hipError_t launch_tile_lists(const uint8_t* mask, int64_t mask_bh, int nQ, int nK, int q_block, int k_block, int n_qt,
+                             int n_kt, int n_qs, int32_t* qt_cnt, int32_t* qt_ent, int32_t* kt_cnt, int32_t* kt_ent,
+                             hipStream_t stream) {
+  const int64_t waves = mask_bh * ((int64_t)n_qt + n_kt);
+  const int64_t blocks = (waves + 3) / 4;
+  if (blocks <= 0) return hipSuccess;
+  if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(tile_lists_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, mask, mask_bh, nQ, nK, q_block, k_block,
+                     n_qt, n_kt, n_qs, qt_cnt, qt_ent, kt_cnt, kt_ent);
+  return hipGetLastError();
+}
+
 // Backward statistics, one pass over O and dO: stats[r] = lse[r] * log2(e) and stats[rows + r] = delta[r] =
 // sum_c dO[r, c] * O[r, c] in fp32 (reference: bwd_attend_prep_ker, flex_block_attn_h100.cu:375-379).  The backward
 // kernels exponentiate in base 2, hence the pre-scaled LSE.  16 lanes per row (16 bytes of each operand per lane).

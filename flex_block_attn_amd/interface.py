@@ -26,7 +26,10 @@ HEAD_DIM = 128
 
 @dataclass
 class BlockLists:
-    """Active-block index lists of one block mask (see include/fba.h, fba_mask_compact)."""
+    """Active-block index lists of one block mask (see include/fba.h, fba_mask_compact).
+
+    With `tiled` set the four tensors are tile lists instead (fba_tile_lists: qt_cnt, qt_ent, kt_cnt, kt_ent), which the
+    kernels need when a block size is not a multiple of 128."""
 
     q_cnt: torch.Tensor  # [mask_bh, nQ] int32
     q_idx: torch.Tensor  # [mask_bh, nQ, nK] int32, ascending, -1 padded
@@ -35,9 +38,12 @@ class BlockLists:
     mask_bh: int
     nQ: int
     nK: int
+    tiled: bool = False
 
     def transposed(self):
-        """Lists of the transposed mask (query and key roles swapped); no device work."""
+        """Lists of the transposed mask (query and key roles swapped); no device work.  Block lists only."""
+        if self.tiled:
+            raise ValueError("tile lists cannot be transposed")
         return BlockLists(self.k_cnt, self.k_idx, self.q_cnt, self.q_idx, self.mask_bh, self.nK, self.nQ)
 
 
@@ -72,6 +78,42 @@ def compact_block_mask(block_mask):
     with torch.cuda.device(dev):
         _lib.call("fba_mask_compact", _ptr(m), mask_bh, nQ, nK, _ptr(q_cnt), _ptr(q_idx), _ptr(k_cnt), _ptr(k_idx), _stream())
     return BlockLists(q_cnt, q_idx, k_cnt, k_idx, mask_bh, nQ, nK)
+
+
+def needs_tile_lists(q_block_size, kv_block_size):
+    """The kernels work on 128-row tiles: block sizes that are not multiples of 128 go through tile lists."""
+    return q_block_size % 128 != 0 or kv_block_size % 128 != 0
+
+
+def tile_block_mask(block_mask, q_block_size, kv_block_size):
+    """bool block mask -> tile lists (a BlockLists with `tiled` set), via fba_tile_lists."""
+    if block_mask.dtype != torch.bool:
+        raise TypeError(f"block_mask must be a bool tensor, got {block_mask.dtype}")
+    if block_mask.dim() not in (2, 4):
+        raise ValueError(f"block_mask must have 2 or 4 dimensions, got {block_mask.dim()}")
+    _require_device(block_mask, "block_mask")
+    m = block_mask.contiguous()
+    nQ, nK = m.shape[-2], m.shape[-1]
+    Sq, Skv = nQ * q_block_size, nK * kv_block_size
+    if Sq % 128 or Skv % 128:
+        raise _lib.FbaError(_lib.FBA_ERR_UNSUPPORTED, f"tile lists need sequence lengths that are multiples of 128, got {Sq} and {Skv}")
+    mask_bh = 1 if m.dim() == 2 else m.shape[0] * m.shape[1]
+    i32 = dict(dtype=torch.int32, device=m.device)
+    qt_cnt = torch.empty((mask_bh, Sq // 128), **i32)
+    qt_ent = torch.empty((mask_bh, Sq // 128, nK), **i32)
+    kt_cnt = torch.empty((mask_bh, Skv // 128), **i32)
+    kt_ent = torch.empty((mask_bh, Skv // 128, Sq // 32), **i32)
+    with torch.cuda.device(m.device):
+        _lib.call("fba_tile_lists", _ptr(m), mask_bh, nQ, nK, q_block_size, kv_block_size, _ptr(qt_cnt), _ptr(qt_ent),
+                  _ptr(kt_cnt), _ptr(kt_ent), _stream())
+    return BlockLists(qt_cnt, qt_ent, kt_cnt, kt_ent, mask_bh, nQ, nK, tiled=True)
+
+
+def lists_for(block_mask, q_block_size, kv_block_size):
+    """The list flavour the kernels need for these block sizes."""
+    if needs_tile_lists(q_block_size, kv_block_size):
+        return tile_block_mask(block_mask, q_block_size, kv_block_size)
+    return compact_block_mask(block_mask)
 
 
 def _check_qkv(q, k, v):
@@ -126,6 +168,8 @@ def _check_blocks(q, k, q_block_size, kv_block_size, block_mask):
 def _check_lists(lists, B, Hq, Sq, Skv, q_block_size, kv_block_size):
     if lists.nQ * q_block_size != Sq or lists.nK * kv_block_size != Skv:
         raise ValueError("block lists do not match the sequence lengths and block sizes")
+    if lists.tiled != needs_tile_lists(q_block_size, kv_block_size):
+        raise ValueError("wrong list flavour for these block sizes (see lists_for)")
     if lists.mask_bh not in (1, B * Hq):
         raise ValueError("block lists do not match batch * heads")
 
@@ -138,7 +182,7 @@ def forward_with_lists(q, k, v, q_block_size, kv_block_size, lists):
     lse = torch.empty((B, Hq, Sq, 1), dtype=torch.float32, device=q.device)
     with torch.cuda.device(q.device):
         _lib.call(
-            "fba_fwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(lists.q_cnt), _ptr(lists.q_idx), lists.mask_bh,
+            "fba_fwd_tiled" if lists.tiled else "fba_fwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(lists.q_cnt), _ptr(lists.q_idx), lists.mask_bh,
             B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size, _stream(),
         )
     return o, lse
@@ -163,7 +207,7 @@ def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists)
     stats = torch.empty((2, B, Hq, Sq), dtype=torch.float32, device=q.device)
     with torch.cuda.device(q.device):
         _lib.call(
-            "fba_bwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), _ptr(dq), _ptr(dk), _ptr(dv),
+            "fba_bwd_tiled" if lists.tiled else "fba_bwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), _ptr(dq), _ptr(dk), _ptr(dv),
             _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), lists.mask_bh,
             B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size, _stream(),
         )
@@ -176,7 +220,7 @@ def _flex_block_attn_forward(q, k, v, q_block_size, kv_block_size, block_mask, s
     reference's kernel needs, is accepted and ignored."""
     fine = small_block_mask if use_small_block_mode else block_mask
     _check_blocks(q, k, q_block_size, kv_block_size, fine)
-    lists = compact_block_mask(fine)
+    lists = lists_for(fine, q_block_size, kv_block_size)
     return forward_with_lists(q, k, v, q_block_size, kv_block_size, lists)
 
 
@@ -186,7 +230,10 @@ def _flex_block_attn_backward(q, k, v, o, lse, do, q_block_size, kv_block_size, 
     fine_t = small_block_mask if use_small_block_mode else block_mask
     if fine_t.dim() not in (2, 4):
         raise ValueError(f"block_mask must have 2 or 4 dimensions, got {fine_t.dim()}")
-    lists = compact_block_mask(fine_t).transposed()
+    if needs_tile_lists(q_block_size, kv_block_size):
+        lists = tile_block_mask(fine_t.transpose(-1, -2).contiguous(), q_block_size, kv_block_size)
+    else:
+        lists = compact_block_mask(fine_t).transposed()
     return backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists)
 
 
@@ -197,13 +244,13 @@ class FlexBlockAttnFunc(torch.autograd.Function):
     def forward(ctx, q, k, v, q_block_size, kv_block_size, block_mask, is_grad_enabled):
         _check_blocks(q, k, q_block_size, kv_block_size, block_mask)
         is_grad = is_grad_enabled and any(x.requires_grad for x in [q, k, v])
-        lists = compact_block_mask(block_mask)
+        lists = lists_for(block_mask, q_block_size, kv_block_size)
         o, lse = forward_with_lists(q, k, v, q_block_size, kv_block_size, lists)
         if is_grad:
             ctx.save_for_backward(q, k, v, o, lse, lists.q_cnt, lists.q_idx, lists.k_cnt, lists.k_idx)
             ctx.q_block_size = q_block_size
             ctx.kv_block_size = kv_block_size
-            ctx.list_meta = (lists.mask_bh, lists.nQ, lists.nK)
+            ctx.list_meta = (lists.mask_bh, lists.nQ, lists.nK, lists.tiled)
         return o
 
     @staticmethod

@@ -57,6 +57,7 @@ int32_t fba_mask_compact(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32
  * Forward.  Replaces attn_forward (attn.cpp:29, flex_block_attn_h100.cu:810-1007; kernel :52-318).
  * Writes o (bf16) and lse (fp32, natural log of the row's softmax denominator including the 1/sqrt(128) scale;
  * -inf and o = 0 for a query block with an empty list).  nQ = Sq / q_block, nK = Skv / k_block.
+ * Needs q_block and k_block to be multiples of 128 (otherwise FBA_ERR_UNSUPPORTED: use fba_tile_lists + fba_fwd_tiled).
  */
 int32_t fba_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* q_cnt,
                 const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
@@ -83,6 +84,28 @@ int32_t fba_bwd_dq(const void* q, const void* k, const void* v, const void* d_o,
 int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,
                      const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
                      int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+
+/*
+ * Block sizes that are not multiples of 128 (the reference allows any q_block % 16 == 0 and kv_block % 64 == 0,
+ * flex_block_attn_interface.py:18-20; its kernels handle them with a second, finer mask and -inf fills,
+ * flex_block_attn_h100.cu:166-243, :512-522).  Here the kernels keep their 128-row tiles and consume tile lists whose
+ * entries carry predicates; Sq and Skv must be multiples of 128.
+ *   qt_cnt   [mask_bh, Sq/128]         entries per 128-row query tile
+ *   qt_ent   [mask_bh, Sq/128, nK]     (J << 8) | bits, ascending J; bit g: 16-row group g of the tile selects key block J
+ *   kt_cnt   [mask_bh, Skv/128]        entries per 128-row key tile
+ *   kt_ent   [mask_bh, Skv/128, Sq/32] (s << 8) | bits, ascending s; bit 2w+f: keys 32w..32w+31 of the tile are selected by
+ *                                      rows 16f..16f+15 of the 32-row query slab s
+ * Unused entries are -1.  fba_fwd_tiled / fba_bwd_tiled take these lists and are otherwise fba_fwd / fba_bwd.
+ */
+int32_t fba_tile_lists(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32_t nK, int32_t q_block, int32_t k_block,
+                       int32_t* qt_cnt, int32_t* qt_ent, int32_t* kt_cnt, int32_t* kt_ent, void* hip_stream);
+int32_t fba_fwd_tiled(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* qt_cnt,
+                      const int32_t* qt_ent, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
+                      int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+int32_t fba_bwd_tiled(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                      float* stats, void* dq, void* dk, void* dv, const int32_t* qt_cnt, const int32_t* qt_ent,
+                      const int32_t* kt_cnt, const int32_t* kt_ent, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
+                      int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
 
 /*
  * Tuning knobs for experiments (process-wide).  No knob is defined at present; every name returns FBA_ERR_INVALID.

@@ -70,6 +70,39 @@ def compact_lists(block_mask):
     return q_cnt, q_idx, k_cnt, k_idx
 
 
+def tile_lists(block_mask, q_block, kv_block):
+    """Brute-force tile lists (include/fba.h, fba_tile_lists) of a bool mask [nQ, nK] or [B, H, nQ, nK]: for every
+    128-row query tile the key blocks selected by any of its eight 16-row groups, with one predicate bit per group; for
+    every 128-row key tile the 32-row query slabs that touch it, with one bit per (32-key wave, 16-row half-slab).
+    Everything follows from allowed(i, j) = mask[i // q_block, j // kv_block]."""
+    m = block_mask.detach().cpu().numpy().astype(bool)
+    nQ, nK = m.shape[-2:]
+    m = m.reshape(-1, nQ, nK)
+    M, Sq, Skv = m.shape[0], nQ * q_block, nK * kv_block
+    n_qt, n_kt, n_qs = Sq // 128, Skv // 128, Sq // 32
+    qt_cnt = np.zeros((M, n_qt), np.int32)
+    qt_ent = np.full((M, n_qt, nK), -1, np.int32)
+    kt_cnt = np.zeros((M, n_kt), np.int32)
+    kt_ent = np.full((M, n_kt, n_qs), -1, np.int32)
+    for b in range(M):
+        for T in range(n_qt):
+            for J in range(nK):
+                bits = sum(int(m[b, (128 * T + 16 * g) // q_block, J]) << g for g in range(8))
+                if bits:
+                    qt_ent[b, T, qt_cnt[b, T]] = (J << 8) | bits
+                    qt_cnt[b, T] += 1
+        for U in range(n_kt):
+            for s_ in range(n_qs):
+                bits = 0
+                for w in range(4):
+                    for f in range(2):
+                        bits |= int(m[b, (32 * s_ + 16 * f) // q_block, (128 * U + 32 * w) // kv_block]) << (2 * w + f)
+                if bits:
+                    kt_ent[b, U, kt_cnt[b, U]] = (s_ << 8) | bits
+                    kt_cnt[b, U] += 1
+    return qt_cnt, qt_ent, kt_cnt, kt_ent
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # restatement 1: explicit formula
 # ---------------------------------------------------------------------------------------------------------------

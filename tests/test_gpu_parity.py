@@ -144,6 +144,87 @@ def test_reference_grid(oracle, gpu, seq, heads, qbs, kbs):
     _run_case(oracle, gpu, 1, heads, heads, seq, seq, qbs, kbs, m, seed=seq + heads, peaky=True)
 
 
+def _reference_raw_mask(nQ, nK):
+    """The reference test's pattern on raw block indices, |j - i| < 2 or j == 4 (test/test_flex_block_attn.py:16-38):
+    with query blocks smaller than key blocks most query blocks beyond the diagonal keep only key block 4, or nothing."""
+    i = torch.arange(nQ)[:, None]
+    j = torch.arange(nK)[None, :]
+    return ((j - i).abs() < 2) | (j == 4)
+
+
+TILE_LIST_CASES = [
+    (16, 64, 24, 6, 0.5), (32, 64, 12, 6, 0.3), (64, 64, 6, 6, 0.5), (64, 128, 8, 4, 0.5), (16, 384, 48, 2, 0.2),
+    (48, 192, 8, 2, 0.5), (128, 64, 3, 6, 0.5), (384, 192, 2, 4, 0.6), (256, 64, 1, 4, 0.5), (64, 256, 8, 2, 1.0),
+    (32, 128, 16, 4, 0.0),
+]
+
+
+def test_tile_lists_bit_exact(oracle, gpu):
+    """fba_tile_lists against the brute-force lists derived from allowed(i, j) alone."""
+    import flex_block_attn_amd as fba
+    from flex_block_attn_amd import masks
+
+    for n, (qbs, kbs, nQ, nK, p) in enumerate(TILE_LIST_CASES):
+        for m in (masks.bernoulli_block_mask(nQ, nK, p, 40 + n), (torch.rand((2, 3, nQ, nK), generator=torch.Generator().manual_seed(n)) < p)):
+            got = fba.tile_block_mask(m.to(gpu), qbs, kbs)
+            assert got.tiled
+            want = oracle.tile_lists(m, qbs, kbs)
+            for g, w, name in zip((got.q_cnt, got.q_idx, got.k_cnt, got.k_idx), want, ("qt_cnt", "qt_ent", "kt_cnt", "kt_ent")):
+                assert g.dtype == torch.int32 and tuple(g.shape) == w.shape, (name, g.shape, w.shape)
+                assert (g.cpu().numpy() == w).all(), f"{name} differs for q{qbs} k{kbs} mask {tuple(m.shape)}"
+
+
+@pytest.mark.parametrize("seq,heads", [(768, 1), (1536, 2)])
+@pytest.mark.parametrize("kbs", [64, 128, 256, 384])
+@pytest.mark.parametrize("qbs", [16, 32, 64])
+def test_reference_grid_small_query_blocks(oracle, gpu, seq, heads, qbs, kbs):
+    """The block sizes of the reference's own test grid (q_block 16/32/64 x kv_block 64/128/256/384,
+    test/test_flex_block_attn.py:70-71), its input distribution and its raw mask pattern."""
+    if seq % kbs:
+        pytest.skip("sequence not divisible")
+    nQ, nK = seq // qbs, seq // kbs
+    m = _reference_raw_mask(nQ, nK)[None, None].expand(1, heads, nQ, nK).contiguous()
+    _run_case(oracle, gpu, 1, heads, heads, seq, seq, qbs, kbs, m, seed=seq + qbs + kbs, peaky=True)
+
+
+@pytest.mark.parametrize("qbs,kbs,Sq,Skv", [(128, 64, 512, 384), (384, 192, 768, 768), (64, 192, 256, 384), (48, 192, 384, 384),
+                                            (16, 64, 128, 128), (256, 64, 512, 256), (80, 320, 640, 640)])
+def test_block_sizes_off_the_tile_grid(oracle, gpu, qbs, kbs, Sq, Skv):
+    """Random masks per head, GQA, block edges that fall inside the kernels' 128-row tiles and 32-row slabs."""
+    from flex_block_attn_amd import masks
+
+    nQ, nK = Sq // qbs, Skv // kbs
+    m = torch.rand((2, 4, nQ, nK), generator=torch.Generator().manual_seed(qbs + kbs)) < 0.5
+    m[..., 0, :] = False  # a query block with nothing selected
+    m[..., :, nK - 1] = False  # a key block nobody selects
+    m[..., nQ - 1, 0] = True
+    _run_case(oracle, gpu, 2, 4, 2, Sq, Skv, qbs, kbs, m, seed=qbs * 7 + kbs)
+
+
+def test_small_block_private_entry_points(oracle, gpu):
+    """use_small_block_mode: the fine mask is the one that counts, the pooled one is ignored
+    (flex_block_attn_interface.py:38-66, :85-86 for the transposed masks of backward)."""
+    import flex_block_attn_amd as fba
+
+    B, H, S, qbs, kbs = 1, 2, 512, 32, 128
+    q, k, v, do = oracle.seeded_qkv(B, H, H, S, S, seed=66)
+    qb, kb, vb, dob = (t.to(torch.bfloat16) for t in (q, k, v, do))
+    fine = torch.rand((S // qbs, S // kbs), generator=torch.Generator().manual_seed(5)) < 0.5
+    fine[:, 0] = True
+    pooled = fine.reshape(S // kbs, kbs // qbs, S // kbs).any(1)
+    o_ref, lse_ref = oracle.c_attention_forward(qb, kb, vb, fine, qbs, kbs)
+    g_ref = oracle.c_attention_backward(qb, kb, vb, o_ref, lse_ref, dob, fine, qbs, kbs)
+    qg, kg, vg, dog = (t.to(gpu) for t in (qb, kb, vb, dob))
+    o, lse = fba._flex_block_attn_forward(qg, kg, vg, qbs, kbs, pooled.to(gpu), fine.to(gpu), True)
+    res = {}
+    _check(oracle, o, o_ref, "o", res)
+    assert oracle.error_metrics(lse.reshape(B, H, S), lse_ref)[0] < 5e-3
+    grads = fba._flex_block_attn_backward(qg, kg, vg, o, lse, dog, qbs, kbs, pooled.t().contiguous().to(gpu),
+                                          fine.t().contiguous().to(gpu), True)
+    for n, got, want in zip(("dq", "dk", "dv"), grads, g_ref):
+        _check(oracle, got, want, n, res)
+
+
 def test_rising_scores_exercise_the_lazy_rescale(oracle, gpu):
     """Keys whose magnitude grows along the sequence: the running softmax reference has to be raised again and again,
     also in the middle of a key block, which N(0,1) inputs never cause."""
@@ -207,15 +288,16 @@ def test_lse_and_private_entry_points(oracle, gpu):
         _check(oracle, got, want, n, res)
 
 
-def test_unsupported_block_sizes_fail_loudly(gpu):
-    """Block sizes the operator allows but this build has no kernel for raise; nothing falls back silently."""
+def test_unsupported_shapes_fail_loudly(gpu):
+    """Shapes the operator allows but this build has no kernel for raise; nothing falls back silently: with a block
+    size off the 128 grid the sequence lengths still have to be multiples of 128."""
     import flex_block_attn_amd as fba
     from flex_block_attn_amd import _lib
 
-    q = torch.zeros((1, 1, 256, 128), dtype=torch.bfloat16, device=gpu)
-    m = torch.ones((4, 2), dtype=torch.bool, device=gpu)
+    q = torch.zeros((1, 1, 192, 128), dtype=torch.bfloat16, device=gpu)
+    m = torch.ones((3, 3), dtype=torch.bool, device=gpu)
     with pytest.raises(_lib.FbaError) as ei:
-        fba.flex_block_attn_func(q, q, q, 64, 128, m)
+        fba.flex_block_attn_func(q, q, q, 64, 64, m)
     assert ei.value.code == _lib.FBA_ERR_UNSUPPORTED
 
 

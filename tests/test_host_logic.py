@@ -67,6 +67,14 @@ def test_c_abi_argument_validation(lib):
     # a shape the operator allows but no kernel variant covers yet is reported as such, not computed wrongly
     assert fwd(1, 1, 2, 2, 256, 256, 128, 64, 128) == lib.FBA_ERR_UNSUPPORTED
     assert b"q_block" in h.fba_last_error()
+    # ... and the tile-list entry points take it, as long as the sequence lengths are multiples of 128
+    assert h.fba_fwd_tiled(f, f, f, f, f, f, f, 1, 1, 2, 2, 192, 192, 128, 64, 64, _null()) == lib.FBA_ERR_UNSUPPORTED
+    assert b"multiples of 128" in h.fba_last_error()
+    assert h.fba_fwd_tiled(_null(), f, f, f, f, f, f, 1, 1, 2, 2, 256, 256, 128, 64, 64, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_tile_lists(f, 1, 3, 3, 64, 64, f, f, f, f, _null()) == lib.FBA_ERR_UNSUPPORTED
+    assert h.fba_tile_lists(f, 1, 4, 4, 24, 64, f, f, f, f, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_tile_lists(f, 1, 4, 4, 64, 64, f, _null(), f, f, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_bwd_tiled(*([f] * 14), 1, 1, 2, 2, 256, 256, 128, 64, 96, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_mask_compact(f, 0, 4, 4, f, f, f, f, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_mask_compact(_null(), 1, 4, 4, f, f, f, f, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_bwd_stats(f, f, f, f, 16, 64, _null()) == lib.FBA_ERR_INVALID
@@ -134,9 +142,6 @@ def test_no_cpu_fallback():
 def test_tensor_contract():
     from flex_block_attn_amd.interface import _check_qkv
 
-    class FakeCuda(torch.Tensor):
-        pass
-
     good = torch.zeros((1, 2, 256, 128), dtype=torch.bfloat16)
     with pytest.raises(ValueError, match="GPU tensor"):
         _check_qkv(good, good, good)
@@ -177,3 +182,12 @@ def test_block_lists_transposed_view():
     a, b, c, d = (torch.zeros(1) for _ in range(4))
     t = BlockLists(a, b, c, d, 1, 3, 5).transposed()
     assert t.q_cnt is c and t.q_idx is d and t.k_cnt is a and t.k_idx is b and (t.nQ, t.nK) == (5, 3)
+    with pytest.raises(ValueError, match="transposed"):
+        BlockLists(a, b, c, d, 1, 3, 5, tiled=True).transposed()
+
+
+def test_list_flavour_follows_block_sizes():
+    from flex_block_attn_amd.interface import needs_tile_lists
+
+    assert not needs_tile_lists(128, 128) and not needs_tile_lists(384, 256)
+    assert needs_tile_lists(64, 128) and needs_tile_lists(128, 192) and needs_tile_lists(16, 64)

@@ -229,6 +229,37 @@ def test_compaction_lists(oracle, shape):
             assert (k_idx[b, j, k_cnt[b, j] :] == -1).all()
 
 
+@pytest.mark.parametrize("qbs,kbs,nQ,nK", [(16, 64, 16, 4), (64, 128, 4, 2), (48, 192, 8, 2), (128, 64, 2, 4), (384, 192, 1, 2), (32, 64, 8, 6)])
+def test_tile_lists_describe_the_dense_mask(oracle, qbs, kbs, nQ, nK):
+    """The tile lists, decoded back, must rebuild exactly the element-level mask: every predicate bit stands for a
+    region inside which the dense mask is constant, and regions without an entry are all False."""
+    g = torch.Generator().manual_seed(qbs + kbs)
+    m = torch.rand((2, nQ, nK), generator=g) < 0.45
+    dense = oracle.expand_block_mask(m, qbs, kbs).numpy()
+    qt_cnt, qt_ent, kt_cnt, kt_ent = oracle.tile_lists(m[:, None], qbs, kbs)
+    Sq, Skv = nQ * qbs, nK * kbs
+    for b in range(2):
+        from_q = np.zeros((Sq, Skv), bool)
+        for T in range(Sq // 128):
+            ents = qt_ent[b, T, : qt_cnt[b, T]]
+            assert (qt_ent[b, T, qt_cnt[b, T]:] == -1).all() and (np.diff(ents >> 8) > 0).all()
+            for e in ents:
+                for grp in range(8):
+                    if (e >> grp) & 1:
+                        from_q[128 * T + 16 * grp: 128 * T + 16 * grp + 16, (e >> 8) * kbs: ((e >> 8) + 1) * kbs] = True
+        from_k = np.zeros((Sq, Skv), bool)
+        for U in range(Skv // 128):
+            ents = kt_ent[b, U, : kt_cnt[b, U]]
+            assert (kt_ent[b, U, kt_cnt[b, U]:] == -1).all() and (np.diff(ents >> 8) > 0).all()
+            for e in ents:
+                for w in range(4):
+                    for f in range(2):
+                        if (e >> (2 * w + f)) & 1:
+                            r0, c0 = 32 * (e >> 8) + 16 * f, 128 * U + 32 * w
+                            from_k[r0: r0 + 16, c0: c0 + 32] = True
+        assert (from_q == dense[b]).all() and (from_k == dense[b]).all()
+
+
 def test_golden_fixtures_match_oracle(oracle):
     """The committed fixtures are what the oracle computes today (guards both against drift)."""
     gdir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
