@@ -3,7 +3,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload random|full|sta|ssta] [--no-cpu]
 
-One step = mask compaction + forward + backward (statistics, dK/dV, dQ) on synthetic inputs already resident in HBM.
+One step = mask compaction + forward + backward (statistics, dK/dV, dQ) on synthetic inputs already resident in HBM; the
+ssta workload also builds its mask from q and k inside the step (block means, scores, top-k).
 Default workload: B=1, H=24, S=30720, head_dim 128, bf16, 384-token blocks (80x80), an independent random mask per
 (batch, head) keeping 32 of 80 key blocks per query-block row with the diagonal forced on.
 FLOPs count selected block pairs only: forward 4*Bq*Bk*D, backward 10*Bq*Bk*D per pair.
@@ -52,13 +53,25 @@ def build_workload(name, device):
         mask = masks.sta_3d_block_mask((5, 6, 10), (3, 3, 3), clamp=True)
         desc = "3-D sliding-tile mask: B1 H24 S115200 D128 bf16, 300 tiles of 6x8x8=384 tokens, 3x3x3 tile window (clamped), 2-D mask"
     elif name == "ssta":
-        raise SystemExit("workload 'ssta' needs the GPU mask builder, which this build does not have yet")
+        B, H, S, qbs, kbs = 1, 24, 69120, 128, 384
+        mask = None  # built on the GPU from q and k inside every step
+        desc = ("asymmetric score-driven mask: B1 H24 S69120 D128 bf16, q block 128 (540) x k block 384 (180); mask = key block of the "
+                "diagonal +-1, key block 0, top-16 key blocks by mean-pooled q . mean-pooled k, built on the GPU inside the step")
     else:
         raise SystemExit(f"unknown workload {name}")
     g = torch.Generator(device="cpu").manual_seed(1234)
     shape = (B, H, S, D)
     q, k, v, do = (torch.randn(shape, generator=g, dtype=torch.float32).to(torch.bfloat16).to(device) for _ in range(4))
-    return dict(B=B, H=H, S=S, qbs=qbs, kbs=kbs, mask=mask.to(device), q=q, k=k, v=v, do=do, desc=desc, nnz=int(mask.sum().item()) * (1 if mask.dim() == 4 else B * H))
+    if mask is None:
+        import flex_block_attn_amd as fba
+
+        mask_fn = lambda: fba.create_ssta_mask(q, k, qbs, kbs, topk=16, band=1, sink_blocks=1)
+        mask = mask_fn()
+    else:
+        mask = mask.to(device)
+        mask_fn = None
+    return dict(B=B, H=H, S=S, qbs=qbs, kbs=kbs, mask=mask, mask_fn=mask_fn, q=q, k=k, v=v, do=do, desc=desc,
+                nnz=int(mask.sum().item()) * (1 if mask.dim() == 4 else B * H))
 
 
 def time_events(fn, warmup, iters):
@@ -135,8 +148,10 @@ def main():
     fl_fwd, fl_bwd = 4.0 * pair_flops * nnz, 10.0 * pair_flops * nnz
     log(f"workload: {w['desc']}; nnz block pairs = {nnz}; fwd {fl_fwd * 1e-12:.3f} TFLOP, bwd {fl_bwd * 1e-12:.3f} TFLOP")
 
+    mask_fn = w["mask_fn"]
+
     def step():
-        lists = fba.compact_block_mask(mask)
+        lists = fba.compact_block_mask(mask_fn() if mask_fn else mask)
         o, lse = fba.forward_with_lists(q, k, v, qbs, kbs, lists)
         return fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists)
 
@@ -165,6 +180,12 @@ def main():
         "bwd_dkdv": lambda: _lib.call("fba_bwd_dkdv", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(stats), _ptr(dk), _ptr(dv), _ptr(lists.k_cnt), _ptr(lists.k_idx), *common, _stream()),
         "bwd_dq": lambda: _lib.call("fba_bwd_dq", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(stats), _ptr(dq), _ptr(lists.q_cnt), _ptr(lists.q_idx), *common, _stream()),
     }
+    if mask_fn:
+        q_mean, k_mean = fba.block_mean(q, qbs), fba.block_mean(k, kbs)
+        mask2 = torch.empty_like(mask)
+        kernels["block_mean_q"] = lambda: _lib.call("fba_block_mean", _ptr(q), _ptr(q_mean), B * H, S, qbs, D, _stream())
+        kernels["block_mean_k"] = lambda: _lib.call("fba_block_mean", _ptr(k), _ptr(k_mean), B * H, S, kbs, D, _stream())
+        kernels["ssta_mask"] = lambda: _lib.call("fba_ssta_mask", _ptr(q_mean), _ptr(k_mean), None, _ptr(mask2), B, H, H, S // qbs, S // kbs, qbs, kbs, 16, 1, 1, _stream())
     iters = max(5, args.steps)
     kms = {}
     for name, fn in kernels.items():
@@ -195,6 +216,11 @@ def main():
         "rooflines": rooflines,
         "mask_compaction": compaction,
     }
+    if mask_fn:
+        pooled = 2.0 * B * H * S * D * 2 + 4.0 * B * H * (S // qbs + S // kbs) * D
+        pool_ms = kms["block_mean_q"]["mean_ms"] + kms["block_mean_k"]["mean_ms"]
+        detail["mask_build"] = {"block_mean_ms": pool_ms, "block_mean_algorithmic_bytes": pooled, "block_mean_GB/s": pooled / (pool_ms * 1e-3) * 1e-9,
+                                "ssta_mask_ms": kms["ssta_mask"]["mean_ms"], "peak_GB/s": PEAK_HBM_GBS}
 
     if args.calibrate_copy:
         src = torch.empty(256 * 1024 * 1024, dtype=torch.uint8, device=dev).fill_(1)

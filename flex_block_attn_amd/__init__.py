@@ -11,7 +11,17 @@ from .interface import (
     lists_for,
     tile_block_mask,
 )
-from . import masks
+from . import masks, video
+from .video import (
+    block_mean,
+    create_moba_3d_mask,
+    create_ssta_3d_mask,
+    create_ssta_mask,
+    create_sta_3d_mask,
+    ssta_3d_attention,
+    tile_tokens,
+    untile_tokens,
+)
 
 __all__ = [
     "flex_block_attn_func",
@@ -25,4 +35,13 @@ __all__ = [
     "lists_for",
     "tile_block_mask",
     "masks",
+    "video",
+    "block_mean",
+    "create_ssta_mask",
+    "create_sta_3d_mask",
+    "create_ssta_3d_mask",
+    "create_moba_3d_mask",
+    "ssta_3d_attention",
+    "tile_tokens",
+    "untile_tokens",
 ]

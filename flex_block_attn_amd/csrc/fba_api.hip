@@ -127,6 +127,47 @@ int32_t fba_fwd_tiled(const void* q, const void* k, const void* v, void* o, floa
   return fwd_impl(q, k, v, o, lse, qt_cnt, qt_ent, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream, true);
 }
 
+int32_t fba_block_mean(const void* x, float* out, int64_t n_seq, int32_t S, int32_t block, int32_t head_dim, void* hip_stream) {
+  if (head_dim != 128) return fail(FBA_ERR_INVALID, "head_dim must be 128, got %d", head_dim);
+  if (n_seq <= 0 || S <= 0) return fail(FBA_ERR_INVALID, "n_seq and S must be positive (got %lld %d)", (long long)n_seq, S);
+  if (block <= 0 || block % 16 != 0 || S % block != 0)
+    return fail(FBA_ERR_INVALID, "block (%d) must be a positive multiple of 16 that divides S (%d)", block, S);
+  if (!out) return fail(FBA_ERR_INVALID, "out is null");
+  if (int rc = check_ptrs({{"x", x}})) return rc;
+  hipError_t e = fba::launch_block_mean((const __bf16*)x, out, n_seq * (S / block), block, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "block_mean launch");
+}
+
+int32_t fba_ssta_mask(const float* q_mean, const float* k_mean, const uint8_t* base, uint8_t* mask, int32_t B, int32_t Hq, int32_t Hkv, int32_t nQ,
+                      int32_t nK, int32_t q_block, int32_t k_block, int32_t topk, int32_t band, int32_t sink,
+                      void* hip_stream) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || nQ <= 0 || nK <= 0)
+    return fail(FBA_ERR_INVALID, "B, Hq, Hkv, nQ, nK must be positive (got %d %d %d %d %d)", B, Hq, Hkv, nQ, nK);
+  if (Hq % Hkv != 0) return fail(FBA_ERR_INVALID, "Hq (%d) must be a multiple of Hkv (%d)", Hq, Hkv);
+  if (q_block <= 0 || k_block <= 0) return fail(FBA_ERR_INVALID, "q_block and k_block must be positive");
+  if (topk < 0 || band < -1 || sink < 0) return fail(FBA_ERR_INVALID, "topk, sink must be >= 0 and band >= -1 (got %d %d %d)", topk, sink, band);
+  if (!q_mean || !k_mean || !mask) return fail(FBA_ERR_INVALID, "null pointer argument");
+  if (nK > 1024) return fail(FBA_ERR_UNSUPPORTED, "at most 1024 key blocks are ranked per query block (got %d)", nK);
+  if ((int64_t)B * Hq > 65535) return fail(FBA_ERR_UNSUPPORTED, "B*Hq (%lld) must be at most 65535", (long long)B * Hq);
+  hipError_t e = fba::launch_ssta_mask(q_mean, k_mean, base, mask, (int64_t)B * Hq, Hq, Hkv, nQ, nK, q_block, k_block, topk, band,
+                                       sink, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "ssta_mask launch");
+}
+
+int32_t fba_tile_permute(const void* x, void* out, int64_t n_seq, int32_t T, int32_t H, int32_t W, int32_t tile_t,
+                         int32_t tile_h, int32_t tile_w, int32_t head_dim, int32_t to_tiles, void* hip_stream) {
+  if (head_dim != 128) return fail(FBA_ERR_INVALID, "head_dim must be 128, got %d", head_dim);
+  if (n_seq <= 0 || T <= 0 || H <= 0 || W <= 0 || tile_t <= 0 || tile_h <= 0 || tile_w <= 0)
+    return fail(FBA_ERR_INVALID, "n_seq, grid and tile extents must be positive");
+  if (T % tile_t != 0 || H % tile_h != 0 || W % tile_w != 0)
+    return fail(FBA_ERR_INVALID, "tile (%d, %d, %d) must divide the grid (%d, %d, %d)", tile_t, tile_h, tile_w, T, H, W);
+  if ((int64_t)T * H * W > 0x7fffffffLL) return fail(FBA_ERR_INVALID, "grid too large");
+  if (x == out) return fail(FBA_ERR_INVALID, "x and out must not alias");
+  if (int rc = check_ptrs({{"x", x}, {"out", out}})) return rc;
+  hipError_t e = fba::launch_tile_permute(x, out, n_seq, T, H, W, tile_t, tile_h, tile_w, to_tiles ? 1 : 0, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "tile_permute launch");
+}
+
 int32_t fba_tile_lists(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32_t nK, int32_t q_block, int32_t k_block,
                        int32_t* qt_cnt, int32_t* qt_ent, int32_t* kt_cnt, int32_t* kt_ent, void* hip_stream) {
   if (mask_bh <= 0 || nQ <= 0 || nK <= 0)

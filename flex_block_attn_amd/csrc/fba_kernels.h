@@ -56,6 +56,11 @@ hipError_t launch_mask_compact(const uint8_t* mask, int64_t mask_bh, int nQ, int
 hipError_t launch_tile_lists(const uint8_t* mask, int64_t mask_bh, int nQ, int nK, int q_block, int k_block, int n_qt,
                              int n_kt, int n_qs, int32_t* qt_cnt, int32_t* qt_ent, int32_t* kt_cnt, int32_t* kt_ent,
                              hipStream_t stream);
+hipError_t launch_block_mean(const __bf16* x, float* out, int64_t n_blocks, int block, hipStream_t stream);
+hipError_t launch_ssta_mask(const float* q_mean, const float* k_mean, const uint8_t* base, uint8_t* mask, int64_t BH, int Hq, int Hkv, int nQ,
+                            int nK, int q_block, int k_block, int topk, int band, int sink, hipStream_t stream);
+hipError_t launch_tile_permute(const void* x, void* out, int64_t n_seq, int T, int H, int W, int tT, int tH, int tW,
+                               int to_tiles, hipStream_t stream);
 hipError_t launch_fwd(FwdParams p, hipStream_t stream);
 hipError_t launch_bwd_stats(const __bf16* o, const __bf16* d_o, const float* lse, float* stats, int64_t rows, hipStream_t stream);
 hipError_t launch_bwd_dq(BwdParams p, hipStream_t stream);

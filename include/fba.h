@@ -108,6 +108,28 @@ int32_t fba_bwd_tiled(const void* q, const void* k, const void* v, const void* o
                       int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
 
 /*
+ * Callers' side of the operator for video models.  The reference names these steps but never released them
+ * (create_sta_3d_mask, create_ssta_3d_mask, create_moba_3d_mask, ssta_3d_attention: flex_block_attn/__init__.py:7-12,
+ * README.md:54-55); they are specified here and checked against their own CPU restatement.
+ *
+ * fba_block_mean: out[s, g, :] = mean of rows g*block .. (g+1)*block-1 of x[s], x [n_seq, S, 128] bf16, out
+ *   [n_seq, S/block, 128] fp32.
+ * fba_ssta_mask: mask[b, h, i, j] (bool bytes, [B, Hq, nQ, nK]) = j is one of the `topk` key blocks with the largest
+ *   <q_mean[b,h,i], k_mean[b, h / (Hq/Hkv), j]> (equal scores: lower j first), or |j - (i*q_block)/k_block| <= band, or
+ *   j < sink, or base[i, j] (base: bool bytes [nQ, nK] shared by every (b, h), e.g. a sliding-tile mask; may be null).
+ *   band = -1 switches the band off.  nK <= 1024.
+ * fba_tile_permute: moves 256-byte token rows of x [n_seq, T*H*W, 128] bf16 between raster order of the (T, H, W) grid
+ *   and tile order (tiles of tile_t x tile_h x tile_w tokens, tiles in raster order of the tile grid, tokens in raster
+ *   order inside a tile), so that one tile is one contiguous block of the attention; to_tiles = 0 is the inverse.
+ */
+int32_t fba_block_mean(const void* x, float* out, int64_t n_seq, int32_t S, int32_t block, int32_t head_dim, void* hip_stream);
+int32_t fba_ssta_mask(const float* q_mean, const float* k_mean, const uint8_t* base, uint8_t* mask, int32_t B, int32_t Hq, int32_t Hkv, int32_t nQ,
+                      int32_t nK, int32_t q_block, int32_t k_block, int32_t topk, int32_t band, int32_t sink,
+                      void* hip_stream);
+int32_t fba_tile_permute(const void* x, void* out, int64_t n_seq, int32_t T, int32_t H, int32_t W, int32_t tile_t,
+                         int32_t tile_h, int32_t tile_w, int32_t head_dim, int32_t to_tiles, void* hip_stream);
+
+/*
  * Tuning knobs for experiments (process-wide).  No knob is defined at present; every name returns FBA_ERR_INVALID.
  */
 int32_t fba_set_option(const char* name, int32_t value);

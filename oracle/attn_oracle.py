@@ -103,6 +103,58 @@ def tile_lists(block_mask, q_block, kv_block):
     return qt_cnt, qt_ent, kt_cnt, kt_ent
 
 
+def block_mean(x, block):
+    """(B, H, S, D) -> (B, H, S / block, D) float64 means of consecutive row blocks (include/fba.h, fba_block_mean)."""
+    B, H, S, D = x.shape
+    return x.double().reshape(B, H, S // block, block, D).mean(3)
+
+
+def ssta_scores(q_mean, k_mean):
+    """<q_mean[b,h,i], k_mean[b, h // (Hq/Hkv), j]> in float64 -> (B, Hq, nQ, nK)."""
+    Hq = q_mean.shape[1]
+    return torch.matmul(q_mean.double(), _repeat_heads(k_mean.double(), Hq).transpose(-1, -2))
+
+
+def _repeat_heads(x, Hq):
+    return x if x.shape[1] == Hq else x.repeat_interleave(Hq // x.shape[1], dim=1)
+
+
+def ssta_mask(scores, q_block, kv_block, topk, band, sink, base=None):
+    """Bool (B, H, nQ, nK) by plain loops over rows (include/fba.h, fba_ssta_mask): the `topk` largest scores of each
+    row, ties to the lower index; key blocks within `band` of the one holding the query block's first row; the first
+    `sink` key blocks; `base` [nQ, nK] if given."""
+    sc = scores.numpy()
+    B, H, nQ, nK = sc.shape
+    out = np.zeros((B, H, nQ, nK), bool)
+    for b in range(B):
+        for h in range(H):
+            for i in range(nQ):
+                order = sorted(range(nK), key=lambda j: (-sc[b, h, i, j], j))
+                out[b, h, i, order[: min(topk, nK)]] = True
+                diag = (i * q_block) // kv_block
+                for j in range(nK):
+                    if abs(j - diag) <= band or j < sink:
+                        out[b, h, i, j] = True
+    if base is not None:
+        out |= base.numpy().astype(bool)[None, None]
+    return torch.from_numpy(out)
+
+
+def tile_order(grid, tile):
+    """Raster index of every token, listed in tile order (include/fba.h, fba_tile_permute): x_tiled = x[..., idx, :]."""
+    T, H, W = grid
+    tT, tH, tW = tile
+    idx = []
+    for bt in range(T // tT):
+        for bh in range(H // tH):
+            for bw in range(W // tW):
+                for it in range(tT):
+                    for ih in range(tH):
+                        for iw in range(tW):
+                            idx.append(((bt * tT + it) * H + bh * tH + ih) * W + bw * tW + iw)
+    return torch.tensor(idx, dtype=torch.long)
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # restatement 1: explicit formula
 # ---------------------------------------------------------------------------------------------------------------

@@ -78,6 +78,17 @@ def test_c_abi_argument_validation(lib):
     assert h.fba_mask_compact(f, 0, 4, 4, f, f, f, f, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_mask_compact(_null(), 1, 4, 4, f, f, f, f, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_bwd_stats(f, f, f, f, 16, 64, _null()) == lib.FBA_ERR_INVALID
+    # caller-side helpers
+    assert h.fba_block_mean(f, f, 4, 256, 24, 128, _null()) == lib.FBA_ERR_INVALID and b"multiple of 16" in h.fba_last_error()
+    assert h.fba_block_mean(f, f, 4, 256, 96, 128, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_block_mean(f, f, 4, 256, 64, 64, _null()) == lib.FBA_ERR_INVALID and b"head_dim" in h.fba_last_error()
+    assert h.fba_block_mean(_null(), f, 4, 256, 64, 128, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_ssta_mask(f, f, _null(), f, 1, 3, 2, 4, 4, 128, 128, 2, 1, 1, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_ssta_mask(f, f, _null(), f, 1, 2, 2, 4, 2000, 128, 128, 2, 1, 1, _null()) == lib.FBA_ERR_UNSUPPORTED
+    assert h.fba_ssta_mask(f, f, _null(), _null(), 1, 2, 2, 4, 4, 128, 128, 2, 1, 1, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_ssta_mask(f, f, _null(), f, 1, 2, 2, 4, 4, 128, 128, -1, 1, 1, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_tile_permute(f, _fake(0x2000), 1, 6, 8, 9, 6, 8, 8, 128, 1, _null()) == lib.FBA_ERR_INVALID and b"divide" in h.fba_last_error()
+    assert h.fba_tile_permute(f, f, 1, 6, 8, 8, 6, 8, 8, 128, 1, _null()) == lib.FBA_ERR_INVALID and b"alias" in h.fba_last_error()
     assert h.fba_set_option(b"no_such_knob", 1) == lib.FBA_ERR_INVALID
     with pytest.raises(lib.FbaError) as ei:
         lib.call("fba_set_option", b"no_such_knob", 1)

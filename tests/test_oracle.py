@@ -260,6 +260,42 @@ def test_tile_lists_describe_the_dense_mask(oracle, qbs, kbs, nQ, nK):
         assert (from_q == dense[b]).all() and (from_k == dense[b]).all()
 
 
+def test_ssta_mask_against_library_topk(oracle):
+    """Row sets against torch.topk on distinct scores; counts and forced entries follow from the definition."""
+    g = torch.Generator().manual_seed(12)
+    q = torch.randn((2, 4, 12 * 32, 16), generator=g)
+    k = torch.randn((2, 2, 6 * 64, 16), generator=g)
+    qm, km = oracle.block_mean(q, 32), oracle.block_mean(k, 64)
+    assert torch.allclose(qm[1, 3, 5], q[1, 3, 160:192].double().mean(0))
+    sc = oracle.ssta_scores(qm, km)
+    assert torch.allclose(sc[1, 3, 5, 2], (qm[1, 3, 5] * km[1, 1, 2]).sum())  # q head 3 reads kv head 1
+    topk = 3
+    m = oracle.ssta_mask(sc, 32, 64, topk, band=-1, sink=0)
+    want = torch.zeros_like(m).scatter_(-1, sc.topk(topk, dim=-1).indices, True)
+    assert torch.equal(m, want) and (m.sum(-1) == topk).all()
+    full = oracle.ssta_mask(sc, 32, 64, topk, band=1, sink=1)
+    i = torch.arange(12)[:, None]
+    j = torch.arange(6)[None, :]
+    forced = ((j - i // 2).abs() <= 1) | (j < 1)
+    assert torch.equal(full, m | forced[None, None])
+    base = torch.rand((12, 6), generator=g) < 0.3
+    assert torch.equal(oracle.ssta_mask(sc, 32, 64, topk, -1, 0, base), m | base[None, None])
+    # ties go to the lower index; asking for more blocks than exist selects all of them
+    flat = torch.zeros((1, 1, 2, 5), dtype=torch.float64)
+    assert oracle.ssta_mask(flat, 64, 64, 2, -1, 0)[0, 0].tolist() == [[True, True, False, False, False]] * 2
+    assert oracle.ssta_mask(flat, 64, 64, 9, -1, 0).all()
+
+
+def test_tile_order_is_the_einops_rearrangement(oracle):
+    import einops
+
+    grid, tile = (4, 6, 4), (2, 3, 2)
+    x = torch.arange(4 * 6 * 4)
+    want = einops.rearrange(x, "(nt tt nh th nw tw) -> (nt nh nw tt th tw)", nt=2, tt=2, nh=2, th=3, nw=2, tw=2)
+    idx = oracle.tile_order(grid, tile)
+    assert torch.equal(x[idx], want) and sorted(idx.tolist()) == list(range(96))
+
+
 def test_golden_fixtures_match_oracle(oracle):
     """The committed fixtures are what the oracle computes today (guards both against drift)."""
     gdir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
