@@ -202,3 +202,20 @@ def test_list_flavour_follows_block_sizes():
 
     assert not needs_tile_lists(128, 128) and not needs_tile_lists(384, 256)
     assert needs_tile_lists(64, 128) and needs_tile_lists(128, 192) and needs_tile_lists(16, 64)
+
+
+def test_benchmark_harness_tables(tmp_path):
+    """CSV layout and block selection of the sweep harness follow the reference scripts (utils.py:31-59, :69-92)."""
+    from flex_block_attn_amd import benchmark
+
+    f = tmp_path / "t.csv"
+    benchmark.append_to_csv({"batch_size": 1, "seq_len": 768, "ptm_attn_executes": 0.5}, str(f))
+    benchmark.append_to_csv({"batch_size": 1, "seq_len": 1536, "ptm_attn_executes": 0.7}, str(f))
+    assert f.read_text().splitlines() == ["batch_size,seq_len,ptm_attn_executes", "1,768,0.5", "1,1536,0.7"]
+    q = torch.zeros((1, 1, 3840, 128))
+    sel = benchmark.selected_blocks("random", q, 384, 0.6, seed=0)
+    assert len(sel) == 10 * 6  # sparse_rate is the KEPT fraction in the reference's scripts
+    swa = benchmark.selected_blocks("swa", q, 384, 0.2, seed=0)
+    assert set(swa) == {(i, j) for i in range(10) for j in range(10) if abs(i - j) < 2}
+    assert len(benchmark.selected_blocks("full", q, 384, 0.0, seed=0)) == 100
+    assert benchmark.SEQ_LENS[0] == 11520 and benchmark.SEQ_LENS[-1] == 84480 and benchmark.SPARSE_RATES == (0.2, 0.4, 0.6, 0.8)
