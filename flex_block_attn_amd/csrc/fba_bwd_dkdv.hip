@@ -122,14 +122,25 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
     if (--rem == 0) next_block(); else row_next += kSlab;
   };
 
+  // Operand registers of one slab's S and dP products: the 16 row-major fetches (Q rows, dO rows)
+  struct ScoreOps {
+    bf16x8 q[8], d[8];
+  };
+  auto fetch_score_ops = [&](const char* stage, ScoreOps& o) {
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      o.q[ks] = lds_read_b128(stage, rm.rd[ks]);
+      o.d[ks] = lds_read_b128(stage + kSlabBytes, rm.rd[ks]);
+    }
+  };
   // S and dP of one slab: 16 MFMAs, the two chains interleaved
-  auto scores = [&](const char* stage, f32x16& s, f32x16& dp) {
+  auto scores = [&](const ScoreOps& o, f32x16& s, f32x16& dp) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-      s = mfma32(lds_read_b128(stage, rm.rd[ks]), kreg[ks], s);
-      dp = mfma32(lds_read_b128(stage + kSlabBytes, rm.rd[ks]), vreg[ks], dp);
+      s = mfma32(o.q[ks], kreg[ks], s);
+      dp = mfma32(o.d[ks], vreg[ks], dp);
     }
   };
 
@@ -142,9 +153,26 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
     wait_vmem<0>();
     __syncthreads();
 #pragma unroll
-    for (int ks = 0; ks < 8; ++ks) { pin(kreg[ks]); pin(vreg[ks]); }
+    for (int ks = 0; ks < 8; ++ks) {  // loop-invariant matrix operands live in the accumulation register file
+      asm volatile("" : "+a"(kreg[ks]));
+      asm volatile("" : "+a"(vreg[ks]));
+    }
+    ScoreOps ops;
     f32x16 s_cur, dp_cur;
-    scores(smem, s_cur, dp_cur);
+    fetch_score_ops(smem, ops);
+    scores(ops, s_cur, dp_cur);
+    fetch_score_ops(smem + kStageBytes, ops);  // a single slab: whatever the second buffer holds, never used
+    // statistics of the slab whose P and dS come next: accumulator element 4g + e of half-wave h is query row 8g + 4h + e
+    f32x4 l4[4], d4[4];
+    auto fetch_stats = [&](const char* stage) {
+      const float* st_lds = reinterpret_cast<const float*>(stage + 2 * kSlabBytes);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        l4[g] = *reinterpret_cast<const f32x4*>(st_lds + 8 * g + 4 * h);
+        d4[g] = *reinterpret_cast<const f32x4*>(st_lds + kSlab + 8 * g + 4 * h);
+      }
+    };
+    fetch_stats(smem);
     // tile lists: predicate bits of the slab being computed, from a second walk over the same lists
     int g_cmp = -1, e_cmp = 0, cnt_cmp = 0, bits_cmp = 0;
     ConstIdx idx_cmp = nullptr;
@@ -164,29 +192,36 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
       next_bits();
     }
 
-    // step t (t % 4 == R): P_t, dS_t from (S_t, dP_t) | S_{t+1}, dP_{t+1} from slab t+1 | dV += dO_t^T P_t, dK += Q_t^T dS_t
+    // Step t (ring slot R = t % 4), entered with (S_t, dP_t) in s_cur / dp_cur and the operands of S_{t+1}, dP_{t+1} in
+    // `ops`.  First half: the matrix pipe computes S_{t+1}, dP_{t+1} while the VALU turns (S_t, dP_t) into P_t, dS_t and
+    // the transposed operands of slab t are fetched.  Slab t is dead after that: barrier, request slab t+4 into its
+    // buffer.  Second half: dV += dO_t^T P_t, dK += Q_t^T dS_t while the operands of slab t+2 are fetched.
     auto step = [&](auto ring_c, int t) {
       const int R = ring_of(ring_c);
       const char* stage = smem + R * kStageBytes;
+      bf16x8 adv[2][4], adk[2][4];
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) {
+          const int roff = 16 * j * kRowBytes;
+          adv[j][mb] = cat(lds_read_tr(stage + kSlabBytes, tr.rd[mb][0] + roff), lds_read_tr(stage + kSlabBytes, tr.rd[mb][1] + roff));
+          adk[j][mb] = cat(lds_read_tr(stage, tr.rd[mb][0] + roff), lds_read_tr(stage, tr.rd[mb][1] + roff));
+        }
       f32x16 s_nxt, dp_nxt;
-      scores(smem + ((R + 1) & 3) * kStageBytes, s_nxt, dp_nxt);  // past the last slab: stale data, unused
-      const float* st_lds = reinterpret_cast<const float*>(stage + 2 * kSlabBytes);
+      scores(ops, s_nxt, dp_nxt);  // past the last slab: stale data, unused
       // does this wave's key block select the first / second 16 query rows of the slab?
       const bool on0 = !kTiled || ((bits_cmp >> (2 * wave)) & 1) != 0;
       const bool on1 = !kTiled || ((bits_cmp >> (2 * wave + 1)) & 1) != 0;
-      // accumulator element 4g + e of half-wave h is query row 8g + 4h + e of the slab
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(st_lds + 8 * g + 4 * h);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(st_lds + kSlab + 8 * g + 4 * h);
+      for (int g = 0; g < 4; ++g)
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          float pv = fast_exp2(__builtin_fmaf(s_cur[4 * g + e], c, -l4[e]));
+          float pv = fast_exp2(__builtin_fmaf(s_cur[4 * g + e], c, -l4[g][e]));
           if constexpr (kTiled) pv = (g < 2 ? on0 : on1) ? pv : 0.f;  // a select: inf or NaN of a masked row is discarded
           s_cur[4 * g + e] = pv;
-          dp_cur[4 * g + e] = pv * (dp_cur[4 * g + e] - d4[e]);
+          dp_cur[4 * g + e] = pv * (dp_cur[4 * g + e] - d4[g][e]);
         }
-      }
       bf16x8 pk[2], dsk[2];
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
@@ -196,22 +231,48 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
                        dp_cur[8 * j + 5], dp_cur[8 * j + 6], dp_cur[8 * j + 7]);
       }
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < 2; ++j) { pin(pk[j]); pin(dsk[j]); }  // computed here, not next to their use after the barrier
+      // issue order of this half, sixteen times: one matrix instruction, two of the 32 transposing fetches, five of the 80
+      // vector instructions.  A wave can have 15 LDS fetches in flight at most (the counter is four bits wide), so fetches
+      // are spread between the matrix instructions instead of being issued in one batch that would block the wave.
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb) {
-          const int roff = 16 * j * kRowBytes;
-          const bf16x8 adv = cat(lds_read_tr(stage + kSlabBytes, tr.rd[mb][0] + roff), lds_read_tr(stage + kSlabBytes, tr.rd[mb][1] + roff));
-          acc_v[mb] = mfma32(adv, pk[j], acc_v[mb]);
-          const bf16x8 adk = cat(lds_read_tr(stage, tr.rd[mb][0] + roff), lds_read_tr(stage, tr.rd[mb][1] + roff));
-          acc_k[mb] = mfma32(adk, dsk[j], acc_k[mb]);
-        }
-      s_cur = s_nxt;
-      dp_cur = dp_nxt;
+      for (int i = 0; i < 16; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+        __builtin_amdgcn_sched_group_barrier(0x002, kTiled ? 6 : 5, 0);
+      }
       if constexpr (kTiled) next_bits();
-      // slab t+2 must have landed (first read in step t+1); the five copies of slab t+3 may still fly
+      __builtin_amdgcn_sched_barrier(0);
+      // slab t+2 must have landed (its operands are fetched below); the five copies of slab t+3 may still fly
       if (t + 3 < nsteps) wait_vmem<5>(); else wait_vmem<0>();
       __syncthreads();
       if (t + 4 < nsteps) copy_next(R);
+      fetch_score_ops(smem + ((R + 2) & 3) * kStageBytes, ops);
+      fetch_stats(smem + ((R + 1) & 3) * kStageBytes);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int mb = 0; mb < 4; ++mb) {
+          acc_v[mb] = mfma32(adv[j][mb], pk[j], acc_v[mb]);
+          acc_k[mb] = mfma32(adk[j][mb], dsk[j], acc_k[mb]);
+        }
+      s_cur = s_nxt;
+      dp_cur = dp_nxt;
+      pin(s_cur);  // the moves out of the accumulation registers happen here, under the products above
+      pin(dp_cur);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {  // the 24 fetches: two after each of the first eight matrix instructions, then one
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 2, 1);
+        __builtin_amdgcn_sched_group_barrier(0x002, 2, 1);
+      }
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 1);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 1);
+        __builtin_amdgcn_sched_group_barrier(0x002, 2, 1);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     };
     if constexpr (kTiled) {
       for (int t = 0; t < nsteps; ++t) step(t & 3, t);  // any step count; ring slot computed at run time
