@@ -99,12 +99,13 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
   const char* dobase = reinterpret_cast<const char*>(p.d_o);
   const char* stbase = reinterpret_cast<const char*>(p.stats);
   int g_cur = -1, e_cur = 0, cnt_cur = 0, rem = 1;
+  bool more = true;  // false once every listed slab has been requested; row_next then stays on the last one
   ConstIdx idx_cur = nullptr;
   int64_t row_next = 0, head_row0 = 0;
   auto next_block = [&]() {  // position row_next on the first row of the next listed query block, if any
     ++e_cur;
     while (e_cur >= cnt_cur) {
-      if (++g_cur >= group) return;
+      if (++g_cur >= group) { more = false; return; }
       const int64_t lr = list_row(g_cur);
       cnt_cur = k_cnt[lr];
       idx_cur = const_idx(p.k_idx + lr * row_len);
@@ -114,11 +115,17 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
     row_next = head_row0 + (kTiled ? (int64_t)(idx_cur[e_cur] >> 8) * kSlab : (int64_t)idx_cur[e_cur] * p.q_block);
     rem = nsub;
   };
-  auto copy_next = [&](int ring) {
+  // Five copies per wave request one slab (Q rows, dO rows, statistics).  Every step issues them, so that the count of
+  // copies in flight is the same at every wait; once the lists are exhausted the last slab is simply requested again,
+  // into a buffer nobody reads any more.
+  auto issue_copy = [&](int ring, int64_t row) {
     const uint32_t dst = ring_dst + ring * kStageBytes;
-    dma.copy(dst, qbase + row_next * kRowBytes);
-    dma.copy(dst + kSlabBytes, dobase + row_next * kRowBytes);
-    dma4(dst + 2 * kSlabBytes, stbase + row_next * 4, stat_off);  // every wave copies the same 256 bytes
+    dma.copy(dst, qbase + row * kRowBytes);
+    dma.copy(dst + kSlabBytes, dobase + row * kRowBytes);
+    dma4(dst + 2 * kSlabBytes, stbase + row * 4, stat_off);  // every wave copies the same 256 bytes
+  };
+  auto advance = [&]() {
+    if (!more) return;
     if (--rem == 0) next_block(); else row_next += kSlab;
   };
 
@@ -148,8 +155,10 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
     e_cur = -1;
     next_block();
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
-      if (j < nsteps) copy_next(j);
+    for (int j = 0; j < 4; ++j) {
+      issue_copy(j, row_next);
+      advance();
+    }
     wait_vmem<0>();
     __syncthreads();
 #pragma unroll
@@ -244,18 +253,21 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
       if constexpr (kTiled) next_bits();
       __builtin_amdgcn_sched_barrier(0);
       // slab t+2 must have landed (its operands are fetched below); the five copies of slab t+3 may still fly
-      if (t + 3 < nsteps) wait_vmem<5>(); else wait_vmem<0>();
+      wait_vmem<5>();
       __syncthreads();
-      if (t + 4 < nsteps) copy_next(R);
+      const int64_t row_copy = row_next;  // slab t+4
+      advance();
       fetch_score_ops(smem + ((R + 2) & 3) * kStageBytes, ops);
       fetch_stats(smem + ((R + 1) & 3) * kStageBytes);
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < 2; ++j) {
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb) {
           acc_v[mb] = mfma32(adv[j][mb], pk[j], acc_v[mb]);
           acc_k[mb] = mfma32(adk[j][mb], dsk[j], acc_k[mb]);
         }
+        if (j == 0) issue_copy(R, row_copy);  // behind eight queued products, not in front of them
+      }
       s_cur = s_nxt;
       dp_cur = dp_nxt;
       pin(s_cur);  // the moves out of the accumulation registers happen here, under the products above
@@ -284,6 +296,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void dkdv_kern
         step(IC<3>{}, t + 3);
       }
     }
+    wait_vmem<0>();  // no copy may still be writing this work-group's LDS when it ends
   }
 
   __bf16* dkrow = p.dk + (krow0 + l32) * kHeadDim;
