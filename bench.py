@@ -37,7 +37,7 @@ def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def build_workload(name, device):
+def build_workload(name, device, inputs="random"):
     from flex_block_attn_amd import masks
 
     if name == "random":
@@ -62,6 +62,9 @@ def build_workload(name, device):
     g = torch.Generator(device="cpu").manual_seed(1234)
     shape = (B, H, S, D)
     q, k, v, do = (torch.randn(shape, generator=g, dtype=torch.float32).to(torch.bfloat16).to(device) for _ in range(4))
+    if inputs == "zeros":  # same instruction stream, no data toggling: shows how much of the time is the power limit
+        for t in (q, k, v, do):
+            t.zero_()
     if mask is None:
         import flex_block_attn_amd as fba
 
@@ -125,6 +128,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="random")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--inputs", choices=["random", "zeros"], default="random",
+                    help="zeros: all-zero q, k, v, dO (a probe of the power limit, not a benchmark figure)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy three times, as the known-size yardstick for rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     args = ap.parse_args()
@@ -140,7 +145,7 @@ def main():
     _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
-    w = build_workload(args.workload, dev)
+    w = build_workload(args.workload, dev, args.inputs)
     B, H, S, qbs, kbs = w["B"], w["H"], w["S"], w["qbs"], w["kbs"]
     q, k, v, do, mask = w["q"], w["k"], w["v"], w["do"], w["mask"]
     nnz = w["nnz"]
@@ -243,7 +248,7 @@ def main():
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "bf16",
-        "data": "synthetic",
+        "data": "synthetic" if args.inputs == "random" else "synthetic, all-zero inputs (power-limit probe, not a benchmark figure)",
         "config": {"workload": w["desc"], "nnz_block_pairs": nnz, "fwd_TFLOP": fl_fwd * 1e-12, "bwd_TFLOP": fl_bwd * 1e-12},
         "roofline": roofline,
         "cpu_baseline": cpu,

@@ -17,6 +17,8 @@ What differs from the reference, deliberately:
 import ctypes
 from dataclasses import dataclass
 
+import math
+
 import torch
 
 from . import _lib
@@ -268,4 +270,25 @@ def flex_block_attn_func(q, k, v, q_block_size, kv_block_size, block_mask):
     q: (batch, heads, q_seq_len, 128) bf16; k, v: (batch, kv_heads, kv_seq_len, 128) bf16; block_mask: bool
     [q_seq_len / q_block_size, kv_seq_len / kv_block_size] or [batch, heads, ...]. Returns o shaped like q.
     """
-    return FlexBlockAttnFunc.apply(q, k, v, q_block_size, kv_block_size, block_mask, torch.is_grad_enabled())
+    pad_q = _pad_rows(q.shape[2], q_block_size, kv_block_size)
+    pad_k = _pad_rows(k.shape[2], kv_block_size, q_block_size)
+    if pad_q == 0 and pad_k == 0:
+        return FlexBlockAttnFunc.apply(q, k, v, q_block_size, kv_block_size, block_mask, torch.is_grad_enabled())
+    # The kernels work on 128-row tiles.  A sequence that is not a multiple of 128 (possible only with block sizes that
+    # are not) is padded with rows that no block selects; the padded query rows come back as zeros and are cut off.
+    _check_blocks(q, k, q_block_size, kv_block_size, block_mask)
+    F = torch.nn.functional
+    qp = F.pad(q, (0, 0, 0, pad_q))
+    kp, vp = F.pad(k, (0, 0, 0, pad_k)), F.pad(v, (0, 0, 0, pad_k))
+    mp = F.pad(block_mask, (0, pad_k // kv_block_size, 0, pad_q // q_block_size), value=False)
+    o = FlexBlockAttnFunc.apply(qp, kp, vp, q_block_size, kv_block_size, mp, torch.is_grad_enabled())
+    return o[:, :, : q.shape[2]]
+
+
+def _pad_rows(seq_len, block, other_block):
+    """Rows to append so that a sequence cut into `block`-row blocks becomes a whole number of 128-row tiles (0 when
+    both block sizes are multiples of 128: the kernels then never see a partial tile)."""
+    if not needs_tile_lists(block, other_block) or seq_len % 128 == 0:
+        return 0
+    unit = block * 128 // math.gcd(block, 128)
+    return -seq_len % unit

@@ -288,16 +288,26 @@ def test_lse_and_private_entry_points(oracle, gpu):
         _check(oracle, got, want, n, res)
 
 
+@pytest.mark.parametrize("qbs,kbs,Sq,Skv", [(64, 64, 192, 192), (16, 64, 80, 320), (48, 192, 144, 576), (128, 64, 384, 192), (32, 128, 96, 128)])
+def test_sequences_that_are_not_whole_tiles(oracle, gpu, qbs, kbs, Sq, Skv):
+    """Sequence lengths that are not multiples of 128 (possible with block sizes that are not): the operator pads them
+    with rows no block selects; results and gradients equal the oracle's on the unpadded problem."""
+    nQ, nK = Sq // qbs, Skv // kbs
+    m = torch.rand((1, 2, nQ, nK), generator=torch.Generator().manual_seed(Sq + Skv)) < 0.6
+    m[..., 0] = True
+    _run_case(oracle, gpu, 1, 2, 2, Sq, Skv, qbs, kbs, m, seed=Sq + 3 * Skv)
+
+
 def test_unsupported_shapes_fail_loudly(gpu):
-    """Shapes the operator allows but this build has no kernel for raise; nothing falls back silently: with a block
-    size off the 128 grid the sequence lengths still have to be multiples of 128."""
+    """The C ABI computes whole 128-row tiles only: asked for anything else it reports so (the Python operator pads
+    before it calls); nothing falls back silently."""
     import flex_block_attn_amd as fba
     from flex_block_attn_amd import _lib
 
     q = torch.zeros((1, 1, 192, 128), dtype=torch.bfloat16, device=gpu)
     m = torch.ones((3, 3), dtype=torch.bool, device=gpu)
     with pytest.raises(_lib.FbaError) as ei:
-        fba.flex_block_attn_func(q, q, q, 64, 64, m)
+        fba._flex_block_attn_forward(q, q, q, 64, 64, m, m, False)
     assert ei.value.code == _lib.FBA_ERR_UNSUPPORTED
 
 

@@ -198,7 +198,11 @@ def test_block_lists_transposed_view():
 
 
 def test_list_flavour_follows_block_sizes():
-    from flex_block_attn_amd.interface import needs_tile_lists
+    from flex_block_attn_amd.interface import _pad_rows, needs_tile_lists
+
+    assert _pad_rows(30720, 384, 384) == 0 and _pad_rows(256, 64, 64) == 0 and _pad_rows(1536, 128, 384) == 0
+    assert _pad_rows(192, 64, 64) == 64 and _pad_rows(80, 16, 64) == 48 and _pad_rows(144, 48, 192) == 240
+    assert _pad_rows(576, 192, 48) == 192 and _pad_rows(192, 64, 128) == 64 and _pad_rows(384, 128, 64) == 0
 
     assert not needs_tile_lists(128, 128) and not needs_tile_lists(384, 256)
     assert needs_tile_lists(64, 128) and needs_tile_lists(128, 192) and needs_tile_lists(16, 64)
