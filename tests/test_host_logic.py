@@ -101,6 +101,11 @@ def test_operator_surface_names():
 
     for name in ("flex_block_attn_func", "_flex_block_attn_forward", "_flex_block_attn_backward"):
         assert getattr(flex_block_attn, name) is getattr(fba, name)
+    from benchmark.utils import utils as ref_path  # the module path the reference's scripts import from
+
+    assert ref_path.create_sparse_mask is fba.masks.create_sparse_mask and ref_path.generate_selected_blocks is fba.masks.generate_selected_blocks
+    q, k, v = ref_path.generate_input(1, 8, 2, 128, "cpu")
+    assert q.shape == (1, 8, 2, 128) and q.dtype == torch.bfloat16 and q.requires_grad
     import inspect
 
     assert list(inspect.signature(fba.flex_block_attn_func).parameters) == ["q", "k", "v", "q_block_size", "kv_block_size", "block_mask"]
