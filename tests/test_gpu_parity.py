@@ -225,6 +225,35 @@ def test_small_block_private_entry_points(oracle, gpu):
         _check(oracle, got, want, n, res)
 
 
+def _random_configs(n, seed):
+    """Seeded draw of legal operator configurations: block sizes from the reference's rule (q % 16, kv % 64, one dividing
+    the other), GQA groups, cross lengths, 2-D or per-(b,h) masks of varying density, some with empty rows or columns."""
+    import random
+
+    rng = random.Random(seed)
+    q_sizes = [16, 32, 48, 64, 96, 128, 192, 256, 384]
+    k_sizes = [64, 128, 192, 256, 384]
+    out = []
+    while len(out) < n:
+        qbs, kbs = rng.choice(q_sizes), rng.choice(k_sizes)
+        if qbs % kbs and kbs % qbs:
+            continue
+        nQ, nK = rng.randint(1, max(1, 768 // qbs)), rng.randint(1, max(1, 768 // kbs))
+        B, Hkv = rng.choice([1, 2]), rng.choice([1, 2])
+        Hq = Hkv * rng.choice([1, 2, 3])
+        out.append((B, Hq, Hkv, nQ * qbs, nK * kbs, qbs, kbs, rng.choice([2, 4]), rng.choice([0.15, 0.5, 0.9, 1.0]), rng.randrange(1 << 30)))
+    return out
+
+
+@pytest.mark.parametrize("cfg", _random_configs(24, seed=2024), ids=lambda c: "B%d_Hq%d_Hkv%d_Sq%d_Skv%d_q%d_k%d_m%d_p%s_%d" % c)
+def test_seeded_random_configurations(oracle, gpu, cfg):
+    B, Hq, Hkv, Sq, Skv, qbs, kbs, mdim, density, seed = cfg
+    g = torch.Generator().manual_seed(seed)
+    shape = (Sq // qbs, Skv // kbs) if mdim == 2 else (B, Hq, Sq // qbs, Skv // kbs)
+    m = torch.rand(shape, generator=g) < density
+    _run_case(oracle, gpu, B, Hq, Hkv, Sq, Skv, qbs, kbs, m, seed=seed % 1000)
+
+
 def test_rising_scores_exercise_the_lazy_rescale(oracle, gpu):
     """Keys whose magnitude grows along the sequence: the running softmax reference has to be raised again and again,
     also in the middle of a key block, which N(0,1) inputs never cause."""
