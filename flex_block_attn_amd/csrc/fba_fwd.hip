@@ -86,9 +86,10 @@ FBA_DEVICE void softmax_reference(FwdState& st, const f32x16& s, bool active) {
   float mx = s[0];
 #pragma unroll
   for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s[r]);
-  mx = max_halves(active ? mx : -INFINITY);
+  mx = active ? mx : -INFINITY;
+  // every half-wave tests the 16 keys it holds; the row maximum over both halves is formed only when the reference rises
   if (__builtin_amdgcn_ballot_w64((mx - st.m_run) * st.c > kLazy) != 0) {
-    const float m_new = fmaxf(st.m_run, mx);
+    const float m_new = fmaxf(st.m_run, max_halves(mx));
     const float alpha = fast_exp2((st.m_run - m_new) * st.c);
     st.m_run = m_new;
 #pragma unroll
