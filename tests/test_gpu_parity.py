@@ -389,3 +389,39 @@ def test_full_size_properties(gpu):
     tok = (perm[:, None] * bs + torch.arange(bs, device=gpu)[None, :]).reshape(-1)
     op, lsep = fba.forward_with_lists(q, k[:, :, tok].contiguous(), v[:, :, tok].contiguous(), bs, bs, fba.compact_block_mask(m[..., perm].contiguous()))
     assert (op.float() - o.float()).abs().max().item() <= 2e-2 and (lsep - lse).abs().max().item() <= 1e-3
+
+
+def test_asymmetric_full_size_properties(gpu):
+    """B1 H6 S69120, q block 128 x k block 384 with the score-driven mask built on the GPU (the asymmetric configuration
+    at its full sequence length, a quarter of its heads): the same oracle-free properties, plus agreement of the selected
+    pairs with the mask's own row structure (every query block keeps block 0, its diagonal band and 16 more at most)."""
+    import flex_block_attn_amd as fba
+
+    B, H, S, qbs, kbs = 1, 6, 69120, 128, 384
+    g = torch.Generator(device="cpu").manual_seed(21)
+    q, k, v, do = (torch.randn((B, H, S, 128), generator=g).to(torch.bfloat16).to(gpu) for _ in range(4))
+    m = fba.create_ssta_mask(q, k, qbs, kbs, topk=16, band=1, sink_blocks=1)
+    nQ, nK = S // qbs, S // kbs
+    assert m.shape == (B, H, nQ, nK) and m[..., 0].all()
+    rows = m.sum(-1)
+    assert int(rows.min()) >= 16 and int(rows.max()) <= 16 + 3 + 1
+    diag = torch.arange(nQ, device=gpu) * qbs // kbs
+    assert m[0, :, torch.arange(nQ, device=gpu), diag].all()
+    lists = fba.compact_block_mask(m)
+
+    o1, _ = fba.forward_with_lists(q, k, torch.ones_like(v), qbs, kbs, lists)
+    assert (o1.float() - 1).abs().max().item() <= 2 ** -7
+    o, lse = fba.forward_with_lists(q, k, v, qbs, kbs, lists)
+    assert torch.isfinite(o).all() and torch.isfinite(lse).all()
+    dq, dk, dv = fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists)
+    dq2, dk2, dv2 = fba.backward_with_lists(q, k, v, o, lse, do * 2, qbs, kbs, lists)
+    for a, b in ((dq, dq2), (dk, dk2), (dv, dv2)):
+        assert torch.isfinite(a).all() and torch.equal(a * 2, b)
+    lhs = (q.float() * dq.float()).sum((-1, -2))
+    rhs = (k.float() * dk.float()).sum((-1, -2))
+    assert ((lhs - rhs).abs() / (q.float() * dq.float()).abs().sum((-1, -2))).max().item() < 2e-3
+    # key blocks that no query block selects get exactly zero gradients
+    unused = ~m.any(-2)  # [B, H, nK]
+    if unused.any():
+        dead = unused.repeat_interleave(kbs, dim=-1)
+        assert dk[dead].abs().max().item() == 0.0 and dv[dead].abs().max().item() == 0.0
