@@ -22,7 +22,6 @@ _c_ptr = ctypes.c_void_p
 SIGNATURES = {
     "fba_version": (_c_i32, []),
     "fba_last_error": (ctypes.c_char_p, []),
-    "fba_set_option": (_c_i32, [ctypes.c_char_p, _c_i32]),
     "fba_mask_compact": (_c_i32, [_c_ptr, _c_i64, _c_i32, _c_i32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr]),
     "fba_fwd": (_c_i32, [_c_ptr] * 7 + [_c_i64] + [_c_i32] * 8 + [_c_ptr]),
     "fba_bwd": (_c_i32, [_c_ptr] * 14 + [_c_i64] + [_c_i32] * 8 + [_c_ptr]),

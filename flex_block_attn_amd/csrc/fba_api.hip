@@ -62,11 +62,6 @@ int32_t fba_version(void) { return 1000; }
 
 const char* fba_last_error(void) { return g_err; }
 
-int32_t fba_set_option(const char* name, int32_t value) {
-  if (name == nullptr) return fail(FBA_ERR_INVALID, "option name is null");
-  return fail(FBA_ERR_INVALID, "unknown option '%s'", name);
-}
-
 int32_t fba_mask_compact(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32_t nK, int32_t* q_cnt, int32_t* q_idx,
                          int32_t* k_cnt, int32_t* k_idx, void* hip_stream) {
   if (mask_bh <= 0 || nQ <= 0 || nK <= 0)
@@ -245,6 +240,10 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_lists(s, tiled, "backward")) return rc;
+  // everything is validated before the first launch, so that a rejected call leaves nothing on the stream
+  if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"o", o}, {"d_o", d_o}, {"dq", dq}, {"dk", dk}, {"dv", dv}})) return rc;
+  if (!lse || !stats || !q_cnt || !q_idx || !k_cnt || !k_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
+  if ((int64_t)B * Hq * Sq >= (1LL << 30)) return fail(FBA_ERR_INVALID, "B*Hq*Sq must be below 2^30");
   if (int rc = fba_bwd_stats(o, d_o, lse, stats, (int64_t)B * Hq * Sq, head_dim, hip_stream)) return rc;
   if (int rc = dkdv_impl(q, k, v, d_o, stats, dk, dv, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block,
                          hip_stream, tiled))

@@ -10,19 +10,13 @@
 //   S^T = K Q^T, dP^T = V dO^T         A = K / V slab rows from LDS (128-bit fetches), B = Q / dO in registers
 //   dS^T = exp2(c S^T - lse2) o (dP^T - delta)
 //   dQ^T += K^T dS^T                   A = K slab through transposing LDS fetches, B = dS^T packed to bf16
-// Software pipeline over 32-key slabs: while the VALU turns (S_t, dP_t) into dS_t, the matrix pipe computes S_{t+1} and
-// dP_{t+1}; the dQ update with dS_t follows.  K and V slabs travel global -> LDS directly into a ring of four
+// Every step handles one 32-key slab: scores, dS, dQ update.  Two waves per SIMD overlap each other (one wave's matrix
+// instructions cover the other's exponentials).  K and V slabs travel global -> LDS directly into a ring of four
 // (K | V) buffers; slab t+4 is requested when slab t is dead, three steps before its first use.
 #include <type_traits>
 
 #include "fba_common.h"
 #include "fba_kernels.h"
-
-// 1: S and dP of slab t+1 are computed during step t (needs both score sets live: more than 256 registers, one wave
-// per SIMD); 0: every step computes its own scores and two waves per SIMD overlap each other.
-#ifndef FBA_DQ_PIPELINED
-#define FBA_DQ_PIPELINED 0
-#endif
 
 namespace fba {
 
@@ -38,14 +32,9 @@ using IC = std::integral_constant<int, N>;
 
 }  // namespace
 
-#if FBA_DQ_PIPELINED
-#define FBA_DQ_OCCUPANCY
-#else
-#define FBA_DQ_OCCUPANCY , amdgpu_waves_per_eu(2, 2)
-#endif
 // kTiled: see the forward kernel (tile lists with a predicate per 16-row group instead of block lists).
 template <bool kTiled>
-__global__ __attribute__((amdgpu_flat_work_group_size(256, 256) FBA_DQ_OCCUPANCY)) void dq_kernel(const BwdParams p) {
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_per_eu(2, 2))) void dq_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];  // ring [4] of (K slab | V slab)
   constexpr int TQ = 128;
 
@@ -134,25 +123,16 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256) FBA_DQ_OCCUPANCY
     __syncthreads();
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) { pin(qreg[ks]); pin(doreg[ks]); }
-#if FBA_DQ_PIPELINED
-    f32x16 s_cur, dp_cur;
-    scores(smem, s_cur, dp_cur);
-#endif
 
     int e_cmp = 0, rem_cmp = nsub;  // list entry of the slab being computed (tile lists: its predicate bits)
     int bits_cmp = kTiled ? idx[0] & 255 : 255;
 
-    // step t (t % 4 == R): dS_t from (S_t, dP_t) | S_{t+1}, dP_{t+1} from slab t+1 | dQ += K_t^T dS_t
+    // step t (t % 4 == R): S_t, dP_t | dS_t | dQ += K_t^T dS_t
     auto step = [&](auto ring_c, int t) {
       constexpr int R = decltype(ring_c)::value;
       const bool active = !kTiled || (bits_cmp & group_bit) != 0;
-#if FBA_DQ_PIPELINED
-      f32x16 s_nxt, dp_nxt;
-      scores(smem + ((R + 1) & 3) * kPairBytes, s_nxt, dp_nxt);  // past the last slab: stale data, unused
-#else
       f32x16 s_cur, dp_cur;
       scores(smem + R * kPairBytes, s_cur, dp_cur);
-#endif
       bf16x8 dsk[2];
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -180,10 +160,6 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256) FBA_DQ_OCCUPANCY
           const bf16x8 a = cat(lds_read_tr(k_t, tr.rd[mb][0] + roff), lds_read_tr(k_t, tr.rd[mb][1] + roff));
           acc[mb] = mfma32(a, dsk[j], acc[mb]);
         }
-#if FBA_DQ_PIPELINED
-      s_cur = s_nxt;
-      dp_cur = dp_nxt;
-#endif
       // slab t+2 must have landed (first read in step t+1); the four copies of slab t+3 may still fly
       if (t + 3 < nsteps) wait_vmem<4>(); else wait_vmem<0>();
       __syncthreads();

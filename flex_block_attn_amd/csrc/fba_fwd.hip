@@ -22,12 +22,6 @@
 #include "fba_common.h"
 #include "fba_kernels.h"
 
-// 1: the softmax denominator is accumulated by two extra MFMAs per step with an all-ones A operand; 0: by VALU
-// additions on the fp32 P values.
-#ifndef FBA_FWD_MFMA_ROWSUM
-#define FBA_FWD_MFMA_ROWSUM 1
-#endif
-
 namespace fba {
 
 namespace {
@@ -73,9 +67,7 @@ FBA_DEVICE void pv_half(FwdState& st, const char* v_half, const bf16x8 (&pk)[2])
       const bf16x8 a = cat(lds_read_tr(v_half, st.tr.rd[mb][0] + roff), lds_read_tr(v_half, st.tr.rd[mb][1] + roff));
       st.acc_o[mb] = mfma32(a, pk[j], st.acc_o[mb]);
     }
-#if FBA_FWD_MFMA_ROWSUM
     st.acc_l = mfma32(st.ones, pk[j], st.acc_l);
-#endif
   }
 }
 
@@ -105,22 +97,11 @@ FBA_DEVICE void softmax_reference(FwdState& st, const f32x16& s, bool active) {
 template <bool kTiled>
 FBA_DEVICE void softmax_exp(FwdState& st, f32x16& s, bf16x8 (&pk)[2], bool active) {
   const float mc = st.m_run * st.c;
-#if FBA_FWD_MFMA_ROWSUM
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     s[r] = fast_exp2(__builtin_fmaf(s[r], st.c, -mc));
     if constexpr (kTiled) s[r] = active ? s[r] : 0.f;
   }
-#else
-  float rs = 0.f;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    s[r] = fast_exp2(__builtin_fmaf(s[r], st.c, -mc));
-    if constexpr (kTiled) s[r] = active ? s[r] : 0.f;
-    rs += s[r];
-  }
-  st.acc_l[0] += rs;  // partial sum of this half-wave's keys
-#endif
 #pragma unroll
   for (int j = 0; j < 2; ++j)
     pk[j] = pack8(s[8 * j + 0], s[8 * j + 1], s[8 * j + 2], s[8 * j + 3], s[8 * j + 4], s[8 * j + 5], s[8 * j + 6], s[8 * j + 7]);
@@ -281,11 +262,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 
   // epilogue: O = O^T / l, LSE = ln2 * (c m + log2 l)
   __bf16* orow = p.o + (qrow0 + l32) * kHeadDim;
-#if FBA_FWD_MFMA_ROWSUM
   const float l = st.acc_l[0];
-#else
-  const float l = sum_halves(st.acc_l[0]);
-#endif
   const float inv = l > 0.f ? 1.f / l : 0.f;
   if (h == 0) p.lse[qrow0 + l32] = l > 0.f ? (st.m_run * st.c + __builtin_log2f(l)) * 0.6931471805599453f : -INFINITY;
 #pragma unroll

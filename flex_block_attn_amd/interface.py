@@ -167,19 +167,29 @@ def _check_blocks(q, k, q_block_size, kv_block_size, block_mask):
         )
 
 
-def _check_lists(lists, B, Hq, Sq, Skv, q_block_size, kv_block_size):
+def _check_lists(lists, q, B, Hq, Sq, Skv, q_block_size, kv_block_size):
+    """The kernels index the list tensors by raw pointer: metadata, dtype, device, layout and exact shapes must fit."""
     if lists.nQ * q_block_size != Sq or lists.nK * kv_block_size != Skv:
         raise ValueError("block lists do not match the sequence lengths and block sizes")
     if lists.tiled != needs_tile_lists(q_block_size, kv_block_size):
         raise ValueError("wrong list flavour for these block sizes (see lists_for)")
     if lists.mask_bh not in (1, B * Hq):
         raise ValueError("block lists do not match batch * heads")
+    M = lists.mask_bh
+    if lists.tiled:
+        shapes = ((M, Sq // 128), (M, Sq // 128, lists.nK), (M, Skv // 128), (M, Skv // 128, Sq // 32))
+    else:
+        shapes = ((M, lists.nQ), (M, lists.nQ, lists.nK), (M, lists.nK), (M, lists.nK, lists.nQ))
+    for name, t, shape in zip(("q_cnt", "q_idx", "k_cnt", "k_idx"), (lists.q_cnt, lists.q_idx, lists.k_cnt, lists.k_idx), shapes):
+        if t.dtype != torch.int32 or t.device != q.device or not t.is_contiguous() or tuple(t.shape) != shape:
+            raise ValueError(f"block lists: {name} must be a contiguous int32 tensor of shape {shape} on {q.device}, "
+                             f"got {tuple(t.shape)} {t.dtype} on {t.device}")
 
 
 def forward_with_lists(q, k, v, q_block_size, kv_block_size, lists):
     """Forward on compacted lists -> (o [B,H,Sq,128] bf16, lse [B,H,Sq,1] fp32)."""
     B, Hq, Hkv, Sq, Skv = _check_qkv(q, k, v)
-    _check_lists(lists, B, Hq, Sq, Skv, q_block_size, kv_block_size)
+    _check_lists(lists, q, B, Hq, Sq, Skv, q_block_size, kv_block_size)
     o = torch.empty_like(q)
     lse = torch.empty((B, Hq, Sq, 1), dtype=torch.float32, device=q.device)
     with torch.cuda.device(q.device):
@@ -193,7 +203,7 @@ def forward_with_lists(q, k, v, q_block_size, kv_block_size, lists):
 def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists):
     """Backward on compacted lists -> (dq, dk, dv), bf16, shaped like q, k, v."""
     B, Hq, Hkv, Sq, Skv = _check_qkv(q, k, v)
-    _check_lists(lists, B, Hq, Sq, Skv, q_block_size, kv_block_size)
+    _check_lists(lists, q, B, Hq, Sq, Skv, q_block_size, kv_block_size)
     if do.dtype != torch.bfloat16:
         do = do.to(torch.bfloat16)
     do = do.contiguous()

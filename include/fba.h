@@ -129,11 +129,6 @@ int32_t fba_ssta_mask(const float* q_mean, const float* k_mean, const uint8_t* b
 int32_t fba_tile_permute(const void* x, void* out, int64_t n_seq, int32_t T, int32_t H, int32_t W, int32_t tile_t,
                          int32_t tile_h, int32_t tile_w, int32_t head_dim, int32_t to_tiles, void* hip_stream);
 
-/*
- * Tuning knobs for experiments (process-wide).  No knob is defined at present; every name returns FBA_ERR_INVALID.
- */
-int32_t fba_set_option(const char* name, int32_t value);
-
 #ifdef __cplusplus
 }
 #endif

@@ -155,6 +155,56 @@ def tile_order(grid, tile):
     return torch.tensor(idx, dtype=torch.long)
 
 
+def sta_window(c, n, w, clamp):
+    """Inclusive range [lo, hi] of key tiles along one axis for the query tile at coordinate c of n, window extent w
+    (odd).  Clipped: the part of [c - w//2, c + w//2] inside the grid.  Clamped: that interval is first slid inwards
+    until it lies inside the grid (then cut to the grid if the axis is shorter than the window), so an interior and a
+    border tile see equally many tiles."""
+    lo, hi = c - w // 2, c + w // 2
+    if clamp:
+        if lo < 0:
+            lo, hi = 0, hi - lo
+        if hi > n - 1:
+            lo, hi = lo - (hi - (n - 1)), n - 1
+    return max(lo, 0), min(hi, n - 1)
+
+
+def sta_3d_mask(tiles, window, clamp=True):
+    """Sliding-tile block mask by plain loops over tile coordinates: tile (t, h, w) has index (t * nh + h) * nw + w
+    (T-major, W-minor); query tile a keeps key tile b iff b lies inside a's window on every axis.  Bool [n, n]."""
+    nt, nh, nw = tiles
+    n = nt * nh * nw
+    out = np.zeros((n, n), bool)
+    for qt in range(nt):
+        t0, t1 = sta_window(qt, nt, window[0], clamp)
+        for qh in range(nh):
+            h0, h1 = sta_window(qh, nh, window[1], clamp)
+            for qw in range(nw):
+                w0, w1 = sta_window(qw, nw, window[2], clamp)
+                a = (qt * nh + qh) * nw + qw
+                for kt in range(t0, t1 + 1):
+                    for kh in range(h0, h1 + 1):
+                        for kw in range(w0, w1 + 1):
+                            out[a, (kt * nh + kh) * nw + kw] = True
+    return torch.from_numpy(out)
+
+
+def sta_token_mask(grid, tile, window, clamp=True):
+    """Token-level sliding-tile mask for a latent in RASTER order, from token coordinates alone: token i =
+    (t * H + h) * W + w attends token j iff the tile holding j lies inside the window of the tile holding i on every
+    axis.  Bool [T*H*W, T*H*W]; independent of any tile enumeration or token permutation."""
+    T, H, W = grid
+    tiles = (T // tile[0], H // tile[1], W // tile[2])
+    coords = np.stack(np.meshgrid(np.arange(T), np.arange(H), np.arange(W), indexing="ij"), -1).reshape(-1, 3)
+    ok = np.ones((len(coords), len(coords)), bool)
+    for ax in range(3):
+        tc = coords[:, ax] // tile[ax]  # tile coordinate of every token along this axis
+        lohi = np.array([sta_window(int(c), tiles[ax], window[ax], clamp) for c in range(tiles[ax])])
+        lo, hi = lohi[tc, 0], lohi[tc, 1]
+        ok &= (tc[None, :] >= lo[:, None]) & (tc[None, :] <= hi[:, None])
+    return torch.from_numpy(ok)
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # restatement 1: explicit formula
 # ---------------------------------------------------------------------------------------------------------------

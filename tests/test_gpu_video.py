@@ -117,3 +117,26 @@ def test_ssta_3d_attention_end_to_end(oracle, gpu):
     for name, got, want in (("o", out, o_ref), ("dq", qg.grad, g_ref[0]), ("dk", kg.grad, g_ref[1]), ("dv", vg.grad, g_ref[2])):
         mabs, rel = oracle.error_metrics(got.float(), want[:, :, inv])
         assert mabs <= 2e-2 and rel <= 1e-2, (name, mabs, rel)
+
+
+@pytest.mark.parametrize("grid,tile,window", [((6, 16, 32), (2, 8, 8), (3, 1, 3)), ((4, 24, 16), (2, 8, 8), (1, 3, 1))])
+def test_sliding_tile_attention_on_raster_latent(oracle, gpu, grid, tile, window):
+    """ssta_3d_attention with the score-driven part switched off (topk 0, no sink) is pure sliding-tile attention.  On a
+    latent in raster order it must equal dense attention under a TOKEN mask built from token coordinates alone
+    (oracle.sta_token_mask): that pins the mask builder's window and axis order and its agreement with the tile
+    permutation's enumeration, neither of which the mask the GPU built is consulted for.  Asymmetric tile grids, so a
+    swapped axis fails."""
+    import flex_block_attn_amd as fba
+
+    S = grid[0] * grid[1] * grid[2]
+    q, k, v, do = oracle.seeded_qkv(1, 2, 2, S, S, seed=S + window[0])
+    qb, kb, vb, dob = (t.to(torch.bfloat16) for t in (q, k, v, do))
+    token_mask = oracle.sta_token_mask(grid, tile, window, clamp=True)
+    o_ref, lse_ref = oracle.dense_attention_explicit(qb, kb, vb, token_mask, 1, 1)
+    g_ref = oracle.dense_attention_backward_explicit(qb, kb, vb, o_ref, lse_ref, dob, token_mask, 1, 1)
+    qg, kg, vg = (t.to(gpu).requires_grad_(True) for t in (qb, kb, vb))
+    out = fba.ssta_3d_attention(qg, kg, vg, grid, tile, window=window, topk=0, sink_blocks=0)
+    out.backward(dob.to(gpu))
+    for name, got, want in (("o", out, o_ref), ("dq", qg.grad, g_ref[0]), ("dk", kg.grad, g_ref[1]), ("dv", vg.grad, g_ref[2])):
+        mabs, rel = oracle.error_metrics(got.float(), want)
+        assert mabs <= 2e-2 and rel <= 1e-2, (name, mabs, rel)

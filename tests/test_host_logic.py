@@ -89,10 +89,18 @@ def test_c_abi_argument_validation(lib):
     assert h.fba_ssta_mask(f, f, _null(), f, 1, 2, 2, 4, 4, 128, 128, -1, 1, 1, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_tile_permute(f, _fake(0x2000), 1, 6, 8, 9, 6, 8, 8, 128, 1, _null()) == lib.FBA_ERR_INVALID and b"divide" in h.fba_last_error()
     assert h.fba_tile_permute(f, f, 1, 6, 8, 8, 6, 8, 8, 128, 1, _null()) == lib.FBA_ERR_INVALID and b"alias" in h.fba_last_error()
-    assert h.fba_set_option(b"no_such_knob", 1) == lib.FBA_ERR_INVALID
+    # FbaError carries the code and the library's message
     with pytest.raises(lib.FbaError) as ei:
-        lib.call("fba_set_option", b"no_such_knob", 1)
-    assert ei.value.code == lib.FBA_ERR_INVALID and "no_such_knob" in ei.value.message
+        lib.call("fba_mask_compact", f, 0, 4, 4, f, f, f, f, _null())
+    assert ei.value.code == lib.FBA_ERR_INVALID and "positive" in ei.value.message
+    # a 4-D mask is indexed by the QUERY head: with grouped kv heads a mask with one slice per kv head is rejected
+    assert h.fba_fwd(f, f, f, f, f, f, f, 2, 1, 4, 2, 256, 256, 128, 128, 128, _null()) == lib.FBA_ERR_INVALID
+    assert b"mask_bh" in h.fba_last_error()
+    assert h.fba_bwd(*([f] * 14), 2, 1, 4, 2, 256, 256, 128, 128, 128, _null()) == lib.FBA_ERR_INVALID and b"mask_bh" in h.fba_last_error()
+    # backward validates every argument before its first launch: a bad gradient pointer is reported, nothing is enqueued
+    bwd_args = [f] * 14
+    bwd_args[7] = _null()  # dq
+    assert h.fba_bwd(*bwd_args, 1, 1, 2, 2, 256, 256, 128, 128, 128, _null()) == lib.FBA_ERR_INVALID and b"dq is null" in h.fba_last_error()
 
 
 def test_operator_surface_names():
@@ -101,6 +109,11 @@ def test_operator_surface_names():
 
     for name in ("flex_block_attn_func", "_flex_block_attn_forward", "_flex_block_attn_backward"):
         assert getattr(flex_block_attn, name) is getattr(fba, name)
+    # the reference's module path (flex_block_attn/__init__.py:1-5 imports from .flex_block_attn_interface)
+    from flex_block_attn.flex_block_attn_interface import FlexBlockAttnFunc, _flex_block_attn_backward, _flex_block_attn_forward, flex_block_attn_func
+
+    assert FlexBlockAttnFunc is fba.FlexBlockAttnFunc and flex_block_attn_func is fba.flex_block_attn_func
+    assert _flex_block_attn_forward is fba._flex_block_attn_forward and _flex_block_attn_backward is fba._flex_block_attn_backward
     from benchmark.utils import utils as ref_path  # the module path the reference's scripts import from
 
     assert ref_path.create_sparse_mask is fba.masks.create_sparse_mask and ref_path.generate_selected_blocks is fba.masks.generate_selected_blocks
@@ -192,6 +205,22 @@ def test_mask_helpers():
     assert int(clipped.sum()) == 5824 and torch.equal(clipped, clipped.t())
 
 
+@pytest.mark.parametrize("tiles,window", [((5, 6, 10), (3, 3, 3)), ((2, 3, 5), (3, 3, 3)), ((1, 2, 2), (3, 3, 3)), ((3, 1, 4), (1, 3, 5)),
+                                          ((4, 2, 3), (5, 1, 3)), ((2, 2, 7), (1, 1, 5))])
+@pytest.mark.parametrize("clamp", [False, True])
+def test_sliding_tile_mask_against_oracle(oracle, tiles, window, clamp):
+    """masks.sta_3d_block_mask against the oracle's loop restatement over (t, h, w) tile coordinates, on asymmetric
+    grids (a swapped axis or another tile enumeration changes the result), with axes shorter than the window."""
+    from flex_block_attn_amd import masks
+
+    got = masks.sta_3d_block_mask(tiles, window, clamp=clamp)
+    want = oracle.sta_3d_mask(tiles, window, clamp=clamp)
+    assert got.dtype == torch.bool and torch.equal(got, want)
+    swapped = oracle.sta_3d_mask((tiles[0], tiles[2], tiles[1]), (window[0], window[2], window[1]), clamp=clamp)
+    if tiles[1] != tiles[2] and (tiles[1] > 1 and tiles[2] > 1):
+        assert not torch.equal(got, swapped)  # the comparison does tell the axes apart
+
+
 def test_block_lists_transposed_view():
     from flex_block_attn_amd.interface import BlockLists
 
@@ -228,3 +257,36 @@ def test_benchmark_harness_tables(tmp_path):
     assert set(swa) == {(i, j) for i in range(10) for j in range(10) if abs(i - j) < 2}
     assert len(benchmark.selected_blocks("full", q, 384, 0.0, seed=0)) == 100
     assert benchmark.SEQ_LENS[0] == 11520 and benchmark.SEQ_LENS[-1] == 84480 and benchmark.SPARSE_RATES == (0.2, 0.4, 0.6, 0.8)
+
+
+def test_block_lists_are_validated_before_any_launch():
+    """A BlockLists whose tensors do not fit the call (shape, dtype, layout) is rejected on the host: the kernels index
+    them by raw pointer."""
+    from flex_block_attn_amd.interface import BlockLists, _check_lists
+
+    q = torch.zeros((1, 2, 256, 128), dtype=torch.bfloat16)
+    i32 = dict(dtype=torch.int32)
+
+    def lists(q_idx_shape=(1, 2, 2), dtype=torch.int32, mask_bh=1):
+        return BlockLists(torch.zeros((mask_bh, 2), **i32), torch.zeros(q_idx_shape, dtype=dtype), torch.zeros((mask_bh, 2), **i32),
+                          torch.zeros((mask_bh, 2, 2), **i32), mask_bh, 2, 2)
+
+    _check_lists(lists(), q, 1, 2, 256, 256, 128, 128)
+    _check_lists(lists((2, 2, 2), mask_bh=2), q, 1, 2, 256, 256, 128, 128)
+    with pytest.raises(ValueError, match="q_idx"):
+        _check_lists(lists((1, 2, 3)), q, 1, 2, 256, 256, 128, 128)
+    with pytest.raises(ValueError, match="q_idx"):
+        _check_lists(lists(dtype=torch.int64), q, 1, 2, 256, 256, 128, 128)
+    with pytest.raises(ValueError, match="batch \\* heads"):
+        _check_lists(lists((3, 2, 2), mask_bh=3), q, 1, 2, 256, 256, 128, 128)
+    bad = lists()
+    bad.k_idx = torch.zeros((1, 2, 4), **i32)[:, :, ::2]
+    with pytest.raises(ValueError, match="k_idx"):
+        _check_lists(bad, q, 1, 2, 256, 256, 128, 128)
+    with pytest.raises(ValueError, match="sequence lengths"):
+        _check_lists(lists(), q, 1, 2, 512, 256, 128, 128)
+    tiled = BlockLists(torch.zeros((1, 2), **i32), torch.zeros((1, 2, 4), **i32), torch.zeros((1, 2), **i32), torch.zeros((1, 2, 8), **i32), 1, 4, 4, tiled=True)
+    _check_lists(tiled, q, 1, 2, 256, 256, 64, 64)
+    tiled.k_idx = torch.zeros((1, 2, 4), **i32)
+    with pytest.raises(ValueError, match="k_idx"):
+        _check_lists(tiled, q, 1, 2, 256, 256, 64, 64)

@@ -296,6 +296,55 @@ def test_tile_order_is_the_einops_rearrangement(oracle):
     assert torch.equal(x[idx], want) and sorted(idx.tolist()) == list(range(96))
 
 
+def test_sliding_tile_mask_restatement(oracle):
+    """Pins oracle.sta_window / sta_3d_mask / sta_token_mask: hand-computed windows, a hand-listed row of an asymmetric
+    grid, the Kronecker product of 1-D band matrices (numpy's kron fixes the T-major, W-minor enumeration: swapping two
+    axes fails it), and the token-level mask against the block mask expanded through the tile permutation."""
+    w = oracle.sta_window
+    assert w(0, 10, 3, True) == (0, 2) and w(9, 10, 3, True) == (7, 9) and w(4, 10, 3, True) == (3, 5)
+    assert w(0, 10, 3, False) == (0, 1) and w(9, 10, 3, False) == (8, 9) and w(4, 10, 3, False) == (3, 5)
+    assert w(1, 10, 5, True) == (0, 4) and w(1, 10, 5, False) == (0, 3) and w(8, 10, 5, True) == (5, 9)
+    assert w(0, 2, 3, True) == (0, 1) and w(1, 2, 3, True) == (0, 1) and w(0, 1, 3, True) == (0, 0) and w(0, 1, 3, False) == (0, 0)
+    assert w(3, 6, 1, True) == (3, 3)
+
+    # tiles (2, 3, 5), clipped 3x3x3 window: tile (1, 2, 3) has index (1*3+2)*5+3 = 28 and keeps t in {0,1}, h in {1,2},
+    # w in {2,3,4}
+    m = oracle.sta_3d_mask((2, 3, 5), (3, 3, 3), clamp=False)
+    want = sorted((t * 3 + h) * 5 + x for t in (0, 1) for h in (1, 2) for x in (2, 3, 4))
+    assert want == [7, 8, 9, 12, 13, 14, 22, 23, 24, 27, 28, 29]
+    assert m[28].nonzero().flatten().tolist() == want
+    # same tile, clamped: t in {0,1} (axis shorter than the window), h slides to {0,1,2}, w in {2,3,4}
+    mc = oracle.sta_3d_mask((2, 3, 5), (3, 3, 3), clamp=True)
+    assert mc[28].nonzero().flatten().tolist() == sorted((t * 3 + h) * 5 + x for t in (0, 1) for h in (0, 1, 2) for x in (2, 3, 4))
+
+    def band(n, wd, clamp):  # 1-D window as a matrix: centre clipped into the grid (clamped) or left alone (clipped)
+        i = np.arange(n)
+        if clamp and n <= wd:
+            return np.ones((n, n), bool)
+        c = np.clip(i, wd // 2, n - 1 - wd // 2) if clamp else i
+        return np.abs(c[:, None] - i[None, :]) <= wd // 2
+
+    for tiles, window in (((2, 3, 5), (3, 3, 3)), ((5, 6, 10), (3, 3, 3)), ((3, 1, 4), (1, 3, 5)), ((4, 2, 3), (5, 1, 3))):
+        for clamp in (False, True):
+            kron = np.kron(np.kron(band(tiles[0], window[0], clamp), band(tiles[1], window[1], clamp)), band(tiles[2], window[2], clamp))
+            got = oracle.sta_3d_mask(tiles, window, clamp)
+            assert np.array_equal(got.numpy(), kron.astype(bool)), (tiles, window, clamp)
+    full = oracle.sta_3d_mask((5, 6, 10), (3, 3, 3), True)
+    assert (full.sum(-1) == 27).all()
+    assert int(oracle.sta_3d_mask((5, 6, 10), (3, 3, 3), False).sum()) == 13 * 16 * 28
+
+    # token-level mask from raster coordinates == block mask expanded to tokens and carried back through the tile order
+    grid, tile, window = (4, 6, 10), (2, 3, 2), (3, 1, 3)
+    tiles = tuple(g // t for g, t in zip(grid, tile))
+    blk = tile[0] * tile[1] * tile[2]
+    idx = oracle.tile_order(grid, tile)
+    for clamp in (False, True):
+        dense_tiled = oracle.expand_block_mask(oracle.sta_3d_mask(tiles, window, clamp), blk, blk)
+        raster = torch.zeros_like(dense_tiled)
+        raster[idx[:, None], idx[None, :]] = dense_tiled
+        assert torch.equal(oracle.sta_token_mask(grid, tile, window, clamp), raster)
+
+
 def test_golden_fixtures_match_oracle(oracle):
     """The committed fixtures are what the oracle computes today (guards both against drift)."""
     gdir = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
