@@ -2,6 +2,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "../../include/fba.h"
 #include "fba_kernels.h"
@@ -267,6 +268,56 @@ int32_t fba_bwd(const void* q, const void* k, const void* v, const void* o, cons
                 float* stats, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
                 const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
                 int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+  return bwd_impl(q, k, v, o, d_o, lse, stats, dq, dk, dv, q_cnt, q_idx, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim,
+                  q_block, k_block, hip_stream, false);
+}
+
+}  // extern "C"
+
+namespace {
+
+// Workspace of fba_bwd_noalloc: the two statistics planes of backward (lse * log2(e), delta) for up to kScratchRows
+// query rows, 32 MiB, held by every GPU the library is loaded on until the process ends.  In host code the array's name
+// is only a handle for hipGetSymbolAddress; kernels get the device address looked up below.
+constexpr int64_t kScratchRows = 1LL << 22;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) float scratch[2 * kScratchRows];
+float* g_scratch_addr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device (each GPU has its own copy at its own address); looked up on the
+// first call on that device.
+int scratch_address(float** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return hip_fail(e, "hipGetDevice");
+  if (dev < 0 || dev >= kMaxDevices) return fail(FBA_ERR_UNSUPPORTED, "device ordinal %d is beyond the %d devices supported", dev, kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_addr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
+    if (ptr == nullptr) return fail(FBA_ERR_HIP, "hipGetSymbolAddress(scratch) returned a null address");
+    g_scratch_addr[dev] = static_cast<float*>(ptr);
+  }
+  *out = g_scratch_addr[dev];
+  return FBA_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t fba_bwd_noalloc(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                        void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx, const int32_t* k_cnt,
+                        const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
+                        int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+  const int64_t rows = (int64_t)B * Hq * Sq;
+  if (B > 0 && Hq > 0 && Sq > 0 && rows > kScratchRows)
+    return fail(FBA_ERR_UNSUPPORTED, "fba_bwd_noalloc: B*Hq*Sq = %lld query rows exceed the built-in workspace of %lld rows; "
+                "call fba_bwd with a caller-owned stats buffer", (long long)rows, (long long)kScratchRows);
+  float* stats = nullptr;
+  if (int rc = scratch_address(&stats)) return rc;
   return bwd_impl(q, k, v, o, d_o, lse, stats, dq, dk, dv, q_cnt, q_idx, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim,
                   q_block, k_block, hip_stream, false);
 }

@@ -86,6 +86,20 @@ int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_
                      int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
 
 /*
+ * fba_bwd without the `stats` argument, for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose host launcher
+ * allocates with torch (flex_block_attn_h100.cu:1077-1093).  The statistics live in a 32 MiB array that is part of the
+ * library's device image, so the call allocates and frees nothing; it serves up to 4 194 304 query rows
+ * (B * Hq * Sq <= 2^22) and returns FBA_ERR_UNSUPPORTED beyond that.  Every call on a GPU uses that GPU's one array:
+ * calls that overlap on one GPU (two streams, two threads) race on it; calls ordered on one stream do not.  Results
+ * are bit-identical to fba_bwd's.
+ */
+int32_t fba_bwd_noalloc(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
+                        void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx, const int32_t* k_cnt,
+                        const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
+                        int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+
+/*
  * Block sizes that are not multiples of 128 (the reference allows any q_block % 16 == 0 and kv_block % 64 == 0,
  * flex_block_attn_interface.py:18-20; its kernels handle them with a second, finer mask and -inf fills,
  * flex_block_attn_h100.cu:166-243, :512-522).  Here the kernels keep their 128-row tiles and consume tile lists whose

@@ -290,3 +290,12 @@ def test_block_lists_are_validated_before_any_launch():
     tiled.k_idx = torch.zeros((1, 2, 4), **i32)
     with pytest.raises(ValueError, match="k_idx"):
         _check_lists(tiled, q, 1, 2, 256, 256, 64, 64)
+
+
+def test_no_alloc_backward_rejects_oversized_problems(lib):
+    """fba_bwd_noalloc serves at most 2^22 query rows from its built-in workspace and says so beyond that, before it
+    touches a device."""
+    h = lib.load()
+    f = _fake()
+    rc = h.fba_bwd_noalloc(*([f] * 13), 1, 1, 64, 64, 128 * 1024, 128 * 1024, 128, 128, 128, _null())
+    assert rc == lib.FBA_ERR_UNSUPPORTED and b"exceed the built-in workspace" in h.fba_last_error()
