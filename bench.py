@@ -27,10 +27,33 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0
 D = 128
 
-# HBM bytes per launch (2 x FETCH_SIZE + WRITE_SIZE KiB, the factors a plain copy of known size gives) from separate
-# rocprofv3 --pmc runs of this script; the counter summary is kept under profiles/.  Only the default workload has been
-# measured; other workloads report null.
-MEASURED_TRAFFIC = {"random": {"fwd": 5.73e9, "bwd_dkdv": 14.90e9, "bwd_dq": 5.90e9}}
+PROFILES = os.path.join(ROOT, "profiles")
+
+
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` from the tracked rocprofv3 counter summary of this workload
+    (profiles/traffic_<workload>.json: 2 x FETCH_SIZE + WRITE_SIZE KiB, scaled by what a plain copy of known size reads),
+    or None when no summary exists or a kernel source is newer than it (a stale figure is worse than none)."""
+    path = os.path.join(PROFILES, f"traffic_{workload}.json")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        rec = json.load(f)
+    csrc = os.path.join(ROOT, "flex_block_attn_amd", "csrc")
+    for src in rec.get("sources", {}).get(kernel, []):
+        if _file_digest(os.path.join(csrc, src)) != rec["digests"].get(src):
+            return None
+    return rec.get("traffic_bytes", {}).get(kernel)
+
+
+def _file_digest(path):
+    import hashlib
+
+    try:
+        with open(path, "rb") as f:
+            return hashlib.sha256(f.read()).hexdigest()[:16]
+    except OSError:
+        return None
 
 
 def log(*a):
@@ -128,6 +151,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="random")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--recompute", action="store_true", help="backward without the dS workspace (fba_bwd: dQ recomputes S and dP)")
     ap.add_argument("--inputs", choices=["random", "zeros"], default="random",
                     help="zeros: all-zero q, k, v, dO (a probe of the power limit, not a benchmark figure)")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -139,7 +163,7 @@ def main():
         raise SystemExit("bench.py needs a GPU")
 
     import flex_block_attn_amd as fba
-    from flex_block_attn_amd import _lib
+    from flex_block_attn_amd import _lib, interface
     from flex_block_attn_amd.interface import _ptr, _stream
 
     _lib.load()
@@ -158,7 +182,7 @@ def main():
     def step():
         lists = fba.compact_block_mask(mask_fn() if mask_fn else mask)
         o, lse = fba.forward_with_lists(q, k, v, qbs, kbs, lists)
-        return fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists)
+        return fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists, hand_over=False if args.recompute else None)
 
     # ---- whole-step timing (the contract's K timed steps) -------------------------------------------------
     for _ in range(args.warmup):
@@ -191,6 +215,15 @@ def main():
         kernels["block_mean_q"] = lambda: _lib.call("fba_block_mean", _ptr(q), _ptr(q_mean), B * H, S, qbs, D, _stream())
         kernels["block_mean_k"] = lambda: _lib.call("fba_block_mean", _ptr(k), _ptr(k_mean), B * H, S, kbs, D, _stream())
         kernels["ssta_mask"] = lambda: _lib.call("fba_ssta_mask", _ptr(q_mean), _ptr(k_mean), None, _ptr(mask2), B, H, H, S // qbs, S // kbs, qbs, kbs, 16, 1, 1, _stream())
+    # the hand-over backward (what the step uses when its workspace fits): dK/dV + dS store, then dQ from the stored dS
+    pairs, ws_bytes = interface.ds_workspace_bytes(lists, B, H, qbs, kbs)
+    hand_over = 0 < ws_bytes <= interface.DS_WORKSPACE_LIMIT_GIB * 2 ** 30 and not args.recompute
+    if hand_over:
+        ds_ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+        ho = (pairs, lists.mask_bh, B, H, H, S, S, D, qbs, kbs)
+        kernels["bwd_dkdv_handover"] = lambda: _lib.call("fba_bwd_dkdv_handover", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(stats), _ptr(dk), _ptr(dv), _ptr(ds_ws), ws_bytes, _ptr(lists.k_cnt), _ptr(lists.k_idx), _ptr(lists.pair_base), *ho, _stream())
+        kernels["bwd_dq_from_ds"] = lambda: _lib.call("fba_bwd_dq_from_ds", _ptr(k), _ptr(ds_ws), ws_bytes, _ptr(dq), _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.q_slot), _ptr(lists.pair_base), *ho, _stream())
+        kernels["pair_slots"] = lambda: _lib.call("fba_pair_slots", _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), lists.mask_bh, lists.nQ, lists.nK, _ptr(lists.pair_base), _ptr(lists.q_slot), _stream())
     iters = max(5, args.steps)
     kms = {}
     for name, fn in kernels.items():
@@ -198,23 +231,36 @@ def main():
         kms[name] = {"mean_ms": sum(ts) / len(ts), "median_ms": statistics.median(ts)}
         log(f"kernel {name}: mean {kms[name]['mean_ms']:.4f} ms, median {kms[name]['median_ms']:.4f} ms")
 
-    # executed MFMA FLOPs per selected block pair: forward 2 products, dK/dV kernel 4 (S, dP, dV, dK), dQ kernel 3
+    # executed MFMA FLOPs per selected block pair: forward 2 products, dK/dV kernel 4 (S, dP, dV, dK), recomputing dQ
+    # kernel 3, dQ from stored dS 1.  The last is bound by memory: it reads every dS element once (2 bytes per
+    # (query, key) of a selected pair), K once and writes dQ.
     kernel_flops = {"fwd": 4.0 * pair_flops * nnz, "bwd_dkdv": 8.0 * pair_flops * nnz, "bwd_dq": 6.0 * pair_flops * nnz}
+    if hand_over:
+        kernel_flops["bwd_dkdv_handover"] = 8.0 * pair_flops * nnz
     rooflines = {}
     for name, fl in kernel_flops.items():
         ach = fl / (kms[name]["mean_ms"] * 1e-3) * 1e-12
         rooflines[name] = {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s", "frac": ach / PEAK_BF16_TFLOPS,
-                           "traffic": MEASURED_TRAFFIC.get(args.workload, {}).get(name), "ms": kms[name]["mean_ms"]}
-    dominant = max(kernel_flops, key=lambda n: kms[n]["mean_ms"])
+                           "traffic": measured_traffic(args.workload, name), "ms": kms[name]["mean_ms"]}
+    if hand_over:
+        ds_bytes = 2.0 * qbs * kbs * nnz + 2.0 * B * H * S * D * 2
+        ach = ds_bytes / (kms["bwd_dq_from_ds"]["mean_ms"] * 1e-3) * 1e-9
+        rooflines["bwd_dq_from_ds"] = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": ach / PEAK_HBM_GBS,
+                                       "traffic": measured_traffic(args.workload, "bwd_dq_from_ds"), "ms": kms["bwd_dq_from_ds"]["mean_ms"]}
+    in_step = [n for n in rooflines if n not in (("bwd_dkdv", "bwd_dq") if hand_over else ("bwd_dkdv_handover", "bwd_dq_from_ds"))]
+    dominant = max(in_step, key=lambda n: kms[n]["mean_ms"])
     roofline = dict(rooflines[dominant])
     roofline["kernel"] = dominant
 
     mask_bytes = mask.numel() + 4 * (2 * nnz // (1 if mask.dim() == 4 else B * H) + lists.mask_bh * (lists.nQ + lists.nK))
     compaction = {"ms": kms["mask_compact"]["mean_ms"], "algorithmic_bytes": mask_bytes, "GB/s": mask_bytes / (kms["mask_compact"]["mean_ms"] * 1e-3) * 1e-9, "peak_GB/s": PEAK_HBM_GBS}
-    bwd_ms = kms["bwd_stats"]["mean_ms"] + kms["bwd_dkdv"]["mean_ms"] + kms["bwd_dq"]["mean_ms"]
+    bwd_recompute_ms = kms["bwd_stats"]["mean_ms"] + kms["bwd_dkdv"]["mean_ms"] + kms["bwd_dq"]["mean_ms"]
+    bwd_ms = kms["bwd_stats"]["mean_ms"] + kms["bwd_dkdv_handover"]["mean_ms"] + kms["bwd_dq_from_ds"]["mean_ms"] if hand_over else bwd_recompute_ms
     detail = {
         "fwd_ms": kms["fwd"]["mean_ms"], "fwd_TFLOP/s": fl_fwd / (kms["fwd"]["mean_ms"] * 1e-3) * 1e-12,
         "bwd_ms": bwd_ms, "bwd_TFLOP/s": fl_bwd / (bwd_ms * 1e-3) * 1e-12,
+        "bwd_path": "dS hand-over (fba_bwd_handover)" if hand_over else "recompute (fba_bwd)",
+        "bwd_recompute_ms": bwd_recompute_ms, "ds_workspace_GB": ws_bytes * 1e-9,
         "fwd+bwd_kernels_TFLOP/s": (fl_fwd + fl_bwd) / ((bwd_ms + kms["fwd"]["mean_ms"]) * 1e-3) * 1e-12,
         "frac_of_bf16_peak": value / PEAK_BF16_TFLOPS,
         "kernels_ms": {n: kms[n]["mean_ms"] for n in kms},

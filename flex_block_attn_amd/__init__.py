@@ -9,6 +9,7 @@ from .interface import (
     flex_block_attn_func,
     forward_with_lists,
     lists_for,
+    number_pairs,
     tile_block_mask,
 )
 from . import masks, video
@@ -33,6 +34,7 @@ __all__ = [
     "forward_with_lists",
     "backward_with_lists",
     "lists_for",
+    "number_pairs",
     "tile_block_mask",
     "masks",
     "video",

@@ -272,6 +272,85 @@ int32_t fba_bwd(const void* q, const void* k, const void* v, const void* o, cons
                   q_block, k_block, hip_stream, false);
 }
 
+int32_t fba_pair_slots(const int32_t* q_cnt, const int32_t* q_idx, const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh,
+                       int32_t nQ, int32_t nK, int32_t* pair_base, int32_t* q_slot, void* hip_stream) {
+  if (mask_bh <= 0 || nQ <= 0 || nK <= 0)
+    return fail(FBA_ERR_INVALID, "mask_bh, nQ, nK must be positive (got %lld %d %d)", (long long)mask_bh, nQ, nK);
+  if (mask_bh * (int64_t)nQ * nK > 0x7fffffffLL) return fail(FBA_ERR_INVALID, "more than 2^31 mask entries");
+  if (!q_cnt || !q_idx || !k_cnt || !k_idx || !pair_base || !q_slot) return fail(FBA_ERR_INVALID, "null pointer argument");
+  hipError_t e = fba::launch_pair_slots(q_cnt, q_idx, k_cnt, k_idx, mask_bh, nQ, nK, pair_base, q_slot, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "pair_slots launch");
+}
+
+// Arguments of the dS hand-over, checked once for all three entry points that take them.
+static int check_handover(const Shape& s, const void* ds_ws, int64_t ds_ws_bytes, const int32_t* pair_base, int64_t n_pairs, const char* what) {
+  if (s.q_block % 128 != 0 || s.k_block % 128 != 0)
+    return fail(FBA_ERR_UNSUPPORTED, "%s: the dS hand-over needs q_block (%d) and k_block (%d) to be multiples of 128", what, s.q_block, s.k_block);
+  if (!pair_base) return fail(FBA_ERR_INVALID, "pair_base is null");
+  if (int rc = check_ptrs({{"ds_ws", ds_ws}})) return rc;
+  if (n_pairs < 0) return fail(FBA_ERR_INVALID, "n_pairs must not be negative");
+  const int64_t need = n_pairs * (int64_t)s.q_block * s.k_block * 2;
+  if (ds_ws_bytes < need)
+    return fail(FBA_ERR_INVALID, "%s: ds_ws holds %lld bytes, %lld pairs of %d x %d need %lld", what, (long long)ds_ws_bytes,
+                (long long)n_pairs, s.q_block, s.k_block, (long long)need);
+  return FBA_OK;
+}
+
+int32_t fba_bwd_dkdv_handover(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,
+                              void* ds_ws, int64_t ds_ws_bytes, const int32_t* k_cnt, const int32_t* k_idx, const int32_t* pair_base,
+                              int64_t n_pairs, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
+                              int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+  const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
+  if (int rc = check_shape(s)) return rc;
+  if (int rc = check_handover(s, ds_ws, ds_ws_bytes, pair_base, n_pairs, "dkdv")) return rc;
+  if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"d_o", d_o}, {"dk", dk}, {"dv", dv}})) return rc;
+  if (!stats || !k_cnt || !k_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
+  if ((int64_t)B * Hq * Sq >= (1LL << 30)) return fail(FBA_ERR_INVALID, "B*Hq*Sq must be below 2^30");
+  fba::BwdParams p{};
+  fill_bwd(p, s);
+  p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.d_o = (const __bf16*)d_o;
+  p.stats = stats; p.dk = (__bf16*)dk; p.dv = (__bf16*)dv; p.k_cnt = k_cnt; p.k_idx = k_idx;
+  p.ds_ws = (__bf16*)ds_ws; p.pair_base = pair_base;
+  hipError_t e = fba::launch_bwd_dkdv(p, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "dkdv (hand-over) launch");
+}
+
+int32_t fba_bwd_dq_from_ds(const void* k, const void* ds_ws, int64_t ds_ws_bytes, void* dq, const int32_t* q_cnt, const int32_t* q_idx,
+                           const int32_t* q_slot, const int32_t* pair_base, int64_t n_pairs, int64_t mask_bh, int32_t B, int32_t Hq,
+                           int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+  const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
+  if (int rc = check_shape(s)) return rc;
+  if (int rc = check_handover(s, ds_ws, ds_ws_bytes, pair_base, n_pairs, "dq")) return rc;
+  if (int rc = check_ptrs({{"k", k}, {"dq", dq}})) return rc;
+  if (!q_cnt || !q_idx || !q_slot) return fail(FBA_ERR_INVALID, "null pointer argument");
+  fba::BwdParams p{};
+  fill_bwd(p, s);
+  p.k = (const __bf16*)k; p.dq = (__bf16*)dq; p.q_cnt = q_cnt; p.q_idx = q_idx;
+  p.ds_ws = (__bf16*)const_cast<void*>(ds_ws); p.pair_base = pair_base; p.q_slot = q_slot;
+  hipError_t e = fba::launch_bwd_dq_from_ds(p, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "dq (from dS) launch");
+}
+
+int32_t fba_bwd_handover(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse, float* stats,
+                         void* ds_ws, int64_t ds_ws_bytes, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
+                         const int32_t* k_cnt, const int32_t* k_idx, const int32_t* pair_base, const int32_t* q_slot, int64_t n_pairs,
+                         int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim,
+                         int32_t q_block, int32_t k_block, void* hip_stream) {
+  const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
+  if (int rc = check_shape(s)) return rc;
+  // everything is validated before the first launch, so that a rejected call leaves nothing on the stream
+  if (int rc = check_handover(s, ds_ws, ds_ws_bytes, pair_base, n_pairs, "backward")) return rc;
+  if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"o", o}, {"d_o", d_o}, {"dq", dq}, {"dk", dk}, {"dv", dv}})) return rc;
+  if (!lse || !stats || !q_cnt || !q_idx || !k_cnt || !k_idx || !q_slot) return fail(FBA_ERR_INVALID, "null pointer argument");
+  if ((int64_t)B * Hq * Sq >= (1LL << 30)) return fail(FBA_ERR_INVALID, "B*Hq*Sq must be below 2^30");
+  if (int rc = fba_bwd_stats(o, d_o, lse, stats, (int64_t)B * Hq * Sq, head_dim, hip_stream)) return rc;
+  if (int rc = fba_bwd_dkdv_handover(q, k, v, d_o, stats, dk, dv, ds_ws, ds_ws_bytes, k_cnt, k_idx, pair_base, n_pairs, mask_bh, B, Hq,
+                                     Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream))
+    return rc;
+  return fba_bwd_dq_from_ds(k, ds_ws, ds_ws_bytes, dq, q_cnt, q_idx, q_slot, pair_base, n_pairs, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim,
+                            q_block, k_block, hip_stream);
+}
+
 }  // extern "C"
 
 namespace {

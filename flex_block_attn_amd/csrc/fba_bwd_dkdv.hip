@@ -42,8 +42,11 @@ using IC = std::integral_constant<int, N>;
 
 // kTiled = false: q_block and k_block are multiples of 128; list entries are query blocks, expanded to q_block/32 slabs.
 // kTiled = true: tile lists; list entries are 32-row query slabs with a predicate per (key group, 16-row half-slab).
-template <bool kTiled>
+// kHandOver (block lists only): every wave also stores the bf16 dS it forms to p.ds_ws (layout: fba_common.h), so that
+// dQ = dS K can be formed later without recomputing S and dP.
+template <bool kTiled, bool kHandOver>
 __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_per_eu(2, 2))) void dkdv_kernel(const BwdParams p) {
+  static_assert(!(kTiled && kHandOver), "dS hand-over works on block lists");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int TK = 128;
 
@@ -160,6 +163,37 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
       next_bits();
       if (par) next_bits();
     }
+    // dS hand-over: (query head of the group, list entry, slab inside the query block) of the slab this wave computes
+    // next, and the pair number of entry 0 of that head's list row
+    int h_g = -1, h_e = -1, h_s = 0, h_cnt = 0;
+    int64_t h_slot0 = 0;
+    const int64_t pair_bytes = (int64_t)p.q_block * p.k_block * 2;
+    const int nsub_k = p.k_block / kSlab;
+    const int t_key = 4 * ((kt * TK - kblk * p.k_block) / TK) + kg;  // this wave's 32-key slab inside the key block
+    const int ho_off0 = ds_unit_store_off(0, lane), ho_off1 = ds_unit_store_off(1, lane);
+    auto ho_next_entry = [&]() {
+      ++h_e;
+      while (h_e >= h_cnt) {
+        if (++h_g >= group) return;
+        const int64_t lr = list_row(h_g);
+        h_cnt = k_cnt[lr];
+        const ConstIdx pb = const_idx(p.pair_base);
+        const int64_t bh = (int64_t)b * p.Hq + hkv * group + h_g;
+        h_slot0 = pb[lr] + (p.mask_bh == 1 ? bh * pb[p.nK] : 0);
+        h_e = 0;
+      }
+    };
+    auto ho_advance = [&](int n) {
+      h_s += n;
+      if (h_s >= nsub) {  // nsub >= 4 > n
+        h_s -= nsub;
+        ho_next_entry();
+      }
+    };
+    if constexpr (kHandOver) {
+      ho_next_entry();
+      ho_advance(par);
+    }
     wait_vmem<0>();
     __syncthreads();
 
@@ -211,6 +245,14 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
         pk[j] = pack8(s[8 * j + 0], s[8 * j + 1], s[8 * j + 2], s[8 * j + 3], s[8 * j + 4], s[8 * j + 5], s[8 * j + 6], s[8 * j + 7]);
         dsk[j] = pack8(dp[8 * j + 0], dp[8 * j + 1], dp[8 * j + 2], dp[8 * j + 3], dp[8 * j + 4], dp[8 * j + 5], dp[8 * j + 6], dp[8 * j + 7]);
       }
+      if constexpr (kHandOver) {
+        char* unit = reinterpret_cast<char*>(p.ds_ws) + (h_slot0 + h_e) * pair_bytes +
+                     (int64_t)((((h_s >> 2) * nsub_k + t_key) * 4 + (h_s & 3)) * kDsUnitBytes);
+        // written once, read once by another kernel much later: streaming stores, so that they do not push the Q / dO
+        // slabs that other work-groups are about to fetch out of L2
+        __builtin_nontemporal_store(dsk[0], reinterpret_cast<bf16x8*>(unit + ho_off0));
+        __builtin_nontemporal_store(dsk[1], reinterpret_cast<bf16x8*>(unit + ho_off1));
+      }
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll
@@ -227,7 +269,10 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     auto step = [&](auto half_c, int s2) {
       if (2 * s2 + par < nslabs) compute(half_c);
       if constexpr (kTiled) { next_bits(); next_bits(); }
-      wait_vmem<0>();   // this wave's copies of the next pair, requested one step ago
+      if constexpr (kHandOver) ho_advance(2);
+      // this wave's copies of the next pair, requested one step ago, must have landed.  The two dS stores of this step are
+      // younger and may still be on their way (the counter covers loads and stores alike and runs down in issue order).
+      if constexpr (kHandOver) wait_vmem<2>(); else wait_vmem<0>();
       __syncthreads();  // everybody is done with this pair and everybody's copies of the next pair have landed
       request_pair(decltype(half_c)::value);
     };
@@ -277,13 +322,12 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
 hipError_t launch_bwd_dkdv(BwdParams p, hipStream_t stream) {
   p.num_items = p.B * p.Hkv * (p.Skv / 128);
   p.items_per_xcd = (p.num_items + kNumXcd - 1) / kNumXcd;
-  const void* fn = p.tiled ? reinterpret_cast<const void*>(&dkdv_kernel<true>) : reinterpret_cast<const void*>(&dkdv_kernel<false>);
-  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
+  const bool hand_over = p.ds_ws != nullptr;
+  if (hand_over && p.tiled) return hipErrorInvalidValue;
+  void (*fn)(const BwdParams) = p.tiled ? &dkdv_kernel<true, false> : hand_over ? &dkdv_kernel<false, true> : &dkdv_kernel<false, false>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
   if (e != hipSuccess) return e;
-  if (p.tiled)
-    hipLaunchKernelGGL(dkdv_kernel<true>, dim3(p.items_per_xcd * kNumXcd), dim3(512), kSmemBytes, stream, p);
-  else
-    hipLaunchKernelGGL(dkdv_kernel<false>, dim3(p.items_per_xcd * kNumXcd), dim3(512), kSmemBytes, stream, p);
+  hipLaunchKernelGGL(fn, dim3(p.items_per_xcd * kNumXcd), dim3(512), kSmemBytes, stream, p);
   return hipGetLastError();
 }
 

@@ -150,6 +150,15 @@ FBA_DEVICE void dma16(uint32_t lds_base, const char* gbase, uint32_t lane_off) {
                : "m0");
 }
 
+// Same copy with the streaming hint: for data that is read exactly once, so that it does not displace what other
+// work-groups are about to re-read from L2.
+FBA_DEVICE void dma16_stream(uint32_t lds_base, const char* gbase, uint32_t lane_off) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+               :
+               : "s"(lds_base), "v"(lane_off), "s"(gbase)
+               : "m0");
+}
+
 // Same for 4 bytes per lane (lane l's dword lands at lds_base + 4 l).
 FBA_DEVICE void dma4(uint32_t lds_base, const char* gbase, uint32_t lane_off) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
@@ -214,5 +223,26 @@ struct TransposedOffsets {
     }
   }
 };
+
+// dS hand-over between the key-major and the query-major backward kernel.  A "unit" is dS of one 32-query slab
+// against 32 keys, 2 KiB of bf16, cut into 256 slots of 8 bytes: slot (key, u) holds dS[4u .. 4u+3][key].  In the
+// key-major kernel lane (key = lane % 32, h = lane / 32) holds, as packed register chunk j, the slots u = 4j + h and
+// u = 4j + 2 + h of its key, 16 bytes.  It stores chunk j at byte offset ds_unit_store_off(j, lane): every 16 lanes
+// fill one contiguous 256 bytes (whole cache lines per pass of the store), and the rotation by 4 h + 8 j inside those
+// 256 bytes spreads the slots that one transposing 64-bit LDS fetch of the query-major kernel touches (4 keys x both h
+// x both halves, for two values of j per half-wave) over all 64 banks.
+FBA_DEVICE int ds_unit_store_off(int j, int lane) {
+  const int key = lane & 31, h = lane >> 5;
+  return j * 1024 + (lane >> 4) * 256 + ((((key & 15) + 4 * h + 8 * j) & 15) << 4);
+}
+// Byte offset of slot (key, u) inside a unit.
+FBA_DEVICE int ds_unit_slot_off(int key, int u) {
+  const int j = u >> 2, half = (u >> 1) & 1, h = u & 1;
+  return j * 1024 + (2 * h + (key >> 4)) * 256 + ((((key & 15) + 4 * h + 8 * j) & 15) << 4) + half * 8;
+}
+// Units of one block pair (q_block x k_block) are ordered for the reader: unit ((tq * (k_block / 32) + t) * 4 + w) is
+// 32-query slab 4 tq + w of the query block against 32-key slab t of the key block, so a 128-row query tile tq reads its
+// whole share of the pair as one ascending stream, 8 KiB (four units, one per wave) per 32-key step.
+constexpr int kDsUnitBytes = 2048;
 
 }  // namespace fba

@@ -49,6 +49,15 @@ struct BwdParams {
   // tiled = 1: q_cnt / q_idx are qt_cnt / qt_ent and k_cnt / k_idx are kt_cnt [mask_bh, Skv/128] /
   // kt_ent [mask_bh, Skv/128, Sq/32] (see tile_lists_kernel)
   int tiled;
+  // dS hand-over (block lists only; null when unused).  The key-major kernel stores dS of every selected block pair
+  // into ds_ws and the query-major kernel reads it back instead of recomputing S and dP.
+  //   pair_base [mask_bh * nK + 1]: exclusive prefix sum of k_cnt; the last entry is the number of pairs in the lists
+  //   q_slot    [mask_bh, nQ, nK]:  pair number of entry e of query block I, i.e. pair_base[m, J] + position of I in
+  //                                 k_idx[m, J, :] for J = q_idx[m, I, e]; -1 beyond q_cnt
+  // Pair n of head bh lives at ds_ws + (n + (mask_bh == 1 ? bh * pairs : 0)) * q_block * k_block * 2 bytes.
+  __bf16* ds_ws;
+  const int32_t* pair_base;
+  const int32_t* q_slot;
 };
 
 hipError_t launch_mask_compact(const uint8_t* mask, int64_t mask_bh, int nQ, int nK, int32_t* q_cnt, int32_t* q_idx,
@@ -65,5 +74,8 @@ hipError_t launch_fwd(FwdParams p, hipStream_t stream);
 hipError_t launch_bwd_stats(const __bf16* o, const __bf16* d_o, const float* lse, float* stats, int64_t rows, hipStream_t stream);
 hipError_t launch_bwd_dq(BwdParams p, hipStream_t stream);
 hipError_t launch_bwd_dkdv(BwdParams p, hipStream_t stream);
+hipError_t launch_bwd_dq_from_ds(BwdParams p, hipStream_t stream);
+hipError_t launch_pair_slots(const int32_t* q_cnt, const int32_t* q_idx, const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh,
+                             int nQ, int nK, int32_t* pair_base, int32_t* q_slot, hipStream_t stream);
 
 }  // namespace fba

@@ -116,6 +116,75 @@ hipError_t launch_tile_lists(const uint8_t* mask, int64_t mask_bh, int nQ, int n
   return hipGetLastError();
 }
 
+// Pair numbering for the dS hand-over of backward.  Every selected (query block, key block) pair gets a number in
+// key-major list order: pair_base = exclusive prefix sum of k_cnt over the flattened (m, J) rows (the last entry is the
+// total), pair (m, J, e) = pair_base[m, J] + e.  q_slot gives the same numbers in query-major list order, so that the
+// query-major kernel finds what the key-major kernel stored: for J = q_idx[m, I, e], q_slot[m, I, e] = pair_base[m, J] +
+// position of I in the ascending row k_idx[m, J, :] (binary search).  Integer work, independent of scheduling.
+__global__ __attribute__((amdgpu_flat_work_group_size(1024, 1024))) void pair_base_kernel(const int32_t* __restrict__ k_cnt, int64_t n,
+                                                                                          int32_t* __restrict__ pair_base) {
+  __shared__ int32_t wave_sum[16];
+  __shared__ int32_t carry_s;
+  const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+  if (tid == 0) carry_s = 0;
+  __syncthreads();
+  for (int64_t t0 = 0; t0 < n; t0 += 1024) {
+    const int64_t t = t0 + tid;
+    const int32_t x = t < n ? k_cnt[t] : 0;
+    int32_t incl = x;  // inclusive scan inside the wave
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int32_t y = __shfl_up(incl, d);
+      if (lane >= d) incl += y;
+    }
+    if (lane == 63) wave_sum[wv] = incl;
+    __syncthreads();
+    int32_t before = carry_s;
+    for (int w = 0; w < wv; ++w) before += wave_sum[w];
+    if (t < n) pair_base[t] = before + incl - x;
+    __syncthreads();
+    if (tid == 1023) carry_s = before + incl;
+    __syncthreads();
+  }
+  if (tid == 0) pair_base[n] = carry_s;
+}
+
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void q_slot_kernel(
+    const int32_t* __restrict__ q_cnt, const int32_t* __restrict__ q_idx, const int32_t* __restrict__ k_cnt,
+    const int32_t* __restrict__ k_idx, const int32_t* __restrict__ pair_base, int64_t mask_bh, int nQ, int nK,
+    int32_t* __restrict__ q_slot) {
+  const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= mask_bh * nQ * nK) return;
+  const int e = (int)(t % nK);
+  const int64_t row = t / nK;  // m * nQ + I
+  const int I = (int)(row % nQ);
+  const int64_t m = row / nQ;
+  int32_t out = -1;
+  if (e < q_cnt[row]) {
+    const int J = q_idx[t];
+    const int64_t krow = m * nK + J;
+    const int32_t* list = k_idx + krow * nQ;
+    int lo = 0, hi = k_cnt[krow] - 1;
+    while (lo < hi) {  // I is in the list: the two orientations describe one mask
+      const int mid = (lo + hi) >> 1;
+      if (list[mid] < I) lo = mid + 1; else hi = mid;
+    }
+    out = pair_base[krow] + lo;
+  }
+  q_slot[t] = out;
+}
+
+hipError_t launch_pair_slots(const int32_t* q_cnt, const int32_t* q_idx, const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh,
+                             int nQ, int nK, int32_t* pair_base, int32_t* q_slot, hipStream_t stream) {
+  const int64_t n = mask_bh * nK, entries = mask_bh * nQ * nK;
+  if (n <= 0 || entries <= 0) return hipSuccess;
+  const int64_t blocks = (entries + 255) / 256;
+  if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(pair_base_kernel, dim3(1), dim3(1024), 0, stream, k_cnt, n, pair_base);
+  hipLaunchKernelGGL(q_slot_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, q_cnt, q_idx, k_cnt, k_idx, pair_base, mask_bh, nQ, nK, q_slot);
+  return hipGetLastError();
+}
+
 // Backward statistics, one pass over O and dO: stats[r] = lse[r] * log2(e) and stats[rows + r] = delta[r] =
 // sum_c dO[r, c] * O[r, c] in fp32 (reference: bwd_attend_prep_ker, flex_block_attn_h100.cu:375-379).  The backward
 // kernels exponentiate in base 2, hence the pre-scaled LSE.  16 lanes per row (16 bytes of each operand per lane).

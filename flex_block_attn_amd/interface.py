@@ -15,9 +15,10 @@ What differs from the reference, deliberately:
     -sqrt(128) times it (flex_block_attn_h100.cu:303-307) and is only ever consumed by its own backward.
 """
 import ctypes
-from dataclasses import dataclass
-
 import math
+import os
+from dataclasses import dataclass
+from typing import Optional
 
 import torch
 
@@ -41,6 +42,17 @@ class BlockLists:
     nQ: int
     nK: int
     tiled: bool = False
+    # pair numbering for the dS hand-over of backward (fba_pair_slots), filled by `number_pairs`
+    pair_base: Optional[torch.Tensor] = None  # [mask_bh * nK + 1] int32; the last entry is the number of listed pairs
+    q_slot: Optional[torch.Tensor] = None     # [mask_bh, nQ, nK] int32
+    _count: Optional[tuple] = None            # (pinned host copy of pair_base[-1], event recorded after the copy)
+
+    def listed_pairs(self):
+        """Number of pairs in the lists (sum of k_cnt), read from the host copy that `number_pairs` requested; waits
+        for that copy only, not for work enqueued after it."""
+        host, event = self._count
+        event.synchronize()
+        return int(host.item())
 
     def transposed(self):
         """Lists of the transposed mask (query and key roles swapped); no device work.  Block lists only."""
@@ -79,7 +91,9 @@ def compact_block_mask(block_mask):
     k_idx = torch.empty((mask_bh, nK, nQ), dtype=torch.int32, device=dev)
     with torch.cuda.device(dev):
         _lib.call("fba_mask_compact", _ptr(m), mask_bh, nQ, nK, _ptr(q_cnt), _ptr(q_idx), _ptr(k_cnt), _ptr(k_idx), _stream())
-    return BlockLists(q_cnt, q_idx, k_cnt, k_idx, mask_bh, nQ, nK)
+    # numbered right away: the host copy of the pair count is then ordered before whatever the caller enqueues next, and
+    # backward finds it without waiting for the forward kernel
+    return number_pairs(BlockLists(q_cnt, q_idx, k_cnt, k_idx, mask_bh, nQ, nK))
 
 
 def needs_tile_lists(q_block_size, kv_block_size):
@@ -200,8 +214,45 @@ def forward_with_lists(q, k, v, q_block_size, kv_block_size, lists):
     return o, lse
 
 
-def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists):
-    """Backward on compacted lists -> (dq, dk, dv), bf16, shaped like q, k, v."""
+def number_pairs(lists):
+    """Pair numbering of block lists for the dS hand-over (fba_pair_slots), kept on `lists`.  The number of listed
+    pairs, which sizes the workspace, is copied to pinned host memory asynchronously; `lists.listed_pairs()` waits for
+    that copy alone."""
+    if lists.tiled:
+        raise ValueError("the dS hand-over works on block lists, not tile lists")
+    if lists.pair_base is None:
+        dev = lists.k_cnt.device
+        pair_base = torch.empty((lists.mask_bh * lists.nK + 1,), dtype=torch.int32, device=dev)
+        q_slot = torch.empty((lists.mask_bh, lists.nQ, lists.nK), dtype=torch.int32, device=dev)
+        host = torch.empty((1,), dtype=torch.int32, pin_memory=True)
+        with torch.cuda.device(dev):
+            _lib.call("fba_pair_slots", _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), lists.mask_bh,
+                      lists.nQ, lists.nK, _ptr(pair_base), _ptr(q_slot), _stream())
+            host.copy_(pair_base[-1:], non_blocking=True)
+            event = torch.cuda.Event()
+            event.record()
+        lists.pair_base, lists.q_slot, lists._count = pair_base, q_slot, (host, event)
+    return lists
+
+
+# Largest dS workspace backward may allocate on its own (GiB); beyond it, or when the allocation fails, backward
+# recomputes S and dP in the dQ kernel instead (fba_bwd).
+DS_WORKSPACE_LIMIT_GIB = float(os.environ.get("FBA_DS_WORKSPACE_LIMIT_GIB", "64"))
+
+
+def ds_workspace_bytes(lists, B, Hq, q_block_size, kv_block_size):
+    """(pairs over all heads, bytes of dS workspace) the hand-over backward needs for these lists."""
+    listed = number_pairs(lists).listed_pairs()
+    pairs = listed * (B * Hq if lists.mask_bh == 1 else 1)
+    return pairs, pairs * q_block_size * kv_block_size * 2
+
+
+def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists, hand_over=None):
+    """Backward on compacted lists -> (dq, dk, dv), bf16, shaped like q, k, v.
+
+    hand_over=True: the key-major kernel stores dS once and dQ is formed from it (fba_bwd_handover, ten products per
+    block pair); False: dQ recomputes S and dP (fba_bwd, fourteen products, no workspace); None: hand over when the
+    lists are block lists and the workspace fits DS_WORKSPACE_LIMIT_GIB and can be allocated."""
     B, Hq, Hkv, Sq, Skv = _check_qkv(q, k, v)
     _check_lists(lists, q, B, Hq, Sq, Skv, q_block_size, kv_block_size)
     if do.dtype != torch.bfloat16:
@@ -217,12 +268,33 @@ def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists)
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)
     stats = torch.empty((2, B, Hq, Sq), dtype=torch.float32, device=q.device)
+    if hand_over and lists.tiled:
+        raise ValueError("the dS hand-over works on block lists (q_block and kv_block multiples of 128)")
+    pairs = ws_bytes = 0
+    ds_ws = None
+    if hand_over or (hand_over is None and not lists.tiled):
+        pairs, ws_bytes = ds_workspace_bytes(lists, B, Hq, q_block_size, kv_block_size)
+        if ws_bytes > 0 and (hand_over or ws_bytes <= DS_WORKSPACE_LIMIT_GIB * 2 ** 30):
+            try:
+                ds_ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=q.device)
+            except torch.OutOfMemoryError:
+                if hand_over:
+                    raise
+    hand_over = ds_ws is not None
     with torch.cuda.device(q.device):
-        _lib.call(
-            "fba_bwd_tiled" if lists.tiled else "fba_bwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), _ptr(dq), _ptr(dk), _ptr(dv),
-            _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), lists.mask_bh,
-            B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size, _stream(),
-        )
+        if hand_over:
+            _lib.call(
+                "fba_bwd_handover", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), _ptr(ds_ws), ws_bytes,
+                _ptr(dq), _ptr(dk), _ptr(dv), _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx),
+                _ptr(lists.pair_base), _ptr(lists.q_slot), pairs, lists.mask_bh,
+                B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size, _stream(),
+            )
+        else:
+            _lib.call(
+                "fba_bwd_tiled" if lists.tiled else "fba_bwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), _ptr(dq), _ptr(dk), _ptr(dv),
+                _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), lists.mask_bh,
+                B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size, _stream(),
+            )
     return dq, dk, dv
 
 
@@ -259,17 +331,16 @@ class FlexBlockAttnFunc(torch.autograd.Function):
         lists = lists_for(block_mask, q_block_size, kv_block_size)
         o, lse = forward_with_lists(q, k, v, q_block_size, kv_block_size, lists)
         if is_grad:
-            ctx.save_for_backward(q, k, v, o, lse, lists.q_cnt, lists.q_idx, lists.k_cnt, lists.k_idx)
+            ctx.save_for_backward(q, k, v, o, lse)
             ctx.q_block_size = q_block_size
             ctx.kv_block_size = kv_block_size
-            ctx.list_meta = (lists.mask_bh, lists.nQ, lists.nK, lists.tiled)
+            ctx.lists = lists  # integer index tensors built here, no part of the autograd graph
         return o
 
     @staticmethod
     def backward(ctx, dout, *args):
-        q, k, v, o, lse, q_cnt, q_idx, k_cnt, k_idx = ctx.saved_tensors
-        lists = BlockLists(q_cnt, q_idx, k_cnt, k_idx, *ctx.list_meta)
-        dq, dk, dv = backward_with_lists(q, k, v, o, lse, dout, ctx.q_block_size, ctx.kv_block_size, lists)
+        q, k, v, o, lse = ctx.saved_tensors
+        dq, dk, dv = backward_with_lists(q, k, v, o, lse, dout, ctx.q_block_size, ctx.kv_block_size, ctx.lists)
         return dq, dk, dv, None, None, None, None
 
 

@@ -86,6 +86,38 @@ int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_
                      int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
 
 /*
+ * Backward with dS handed over in memory.  fba_bwd computes S and dP twice, once in the key-major kernel (dK, dV) and
+ * once in the query-major kernel (dQ), because no kernel may add into rows it does not own.  The reference avoids the
+ * second computation with reducing stores into fp32 dQ (flex_block_attn_h100.cu:707-708); fp32 atomic adds run at
+ * about 1.4 TB/s on this GPU, far too slow for that.  Here the key-major kernel instead stores the bf16 dS of every
+ * selected block pair once into `ds_ws` and a light query-major kernel forms dQ = dS K from it: ten products per pair
+ * instead of fourteen, still no atomics, bit-reproducible, at the price of the workspace.  Block lists only
+ * (q_block and k_block multiples of 128).
+ *   fba_pair_slots   numbers the pairs: pair_base [mask_bh * nK + 1] = exclusive prefix sum of k_cnt (last entry =
+ *                    number of pairs in the lists), q_slot [mask_bh, nQ, nK] = the pair number of every q_idx entry
+ *                    (-1 beyond q_cnt).
+ *   ds_ws            n_pairs * q_block * k_block bf16, 16-byte aligned; n_pairs = selected pairs over all (batch,
+ *                    head): the sum of k_cnt, times B * Hq when mask_bh == 1.  ds_ws_bytes is its size; the caller
+ *                    vouches that n_pairs matches the lists (they live in device memory and are not read back).
+ * Other arguments as fba_bwd; dq, dk, dv agree with fba_bwd's to within bf16 rounding of dS (dk, dv bit for bit).
+ */
+int32_t fba_pair_slots(const int32_t* q_cnt, const int32_t* q_idx, const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh,
+                       int32_t nQ, int32_t nK, int32_t* pair_base, int32_t* q_slot, void* hip_stream);
+int32_t fba_bwd_handover(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse, float* stats,
+                         void* ds_ws, int64_t ds_ws_bytes, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
+                         const int32_t* k_cnt, const int32_t* k_idx, const int32_t* pair_base, const int32_t* q_slot, int64_t n_pairs,
+                         int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim,
+                         int32_t q_block, int32_t k_block, void* hip_stream);
+/* Its two attention stages separately (after fba_bwd_stats), for profiling one kernel at a time. */
+int32_t fba_bwd_dkdv_handover(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,
+                              void* ds_ws, int64_t ds_ws_bytes, const int32_t* k_cnt, const int32_t* k_idx, const int32_t* pair_base,
+                              int64_t n_pairs, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
+                              int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+int32_t fba_bwd_dq_from_ds(const void* k, const void* ds_ws, int64_t ds_ws_bytes, void* dq, const int32_t* q_cnt, const int32_t* q_idx,
+                           const int32_t* q_slot, const int32_t* pair_base, int64_t n_pairs, int64_t mask_bh, int32_t B, int32_t Hq,
+                           int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+
+/*
  * fba_bwd without the `stats` argument, for callers that cannot allocate device memory (code under HIP graph capture,
  * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose host launcher
  * allocates with torch (flex_block_attn_h100.cu:1077-1093).  The statistics live in a 32 MiB array that is part of the

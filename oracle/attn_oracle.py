@@ -70,6 +70,30 @@ def compact_lists(block_mask):
     return q_cnt, q_idx, k_cnt, k_idx
 
 
+def pair_numbering(q_cnt, q_idx, k_cnt, k_idx):
+    """Numbers of the selected block pairs in key-major list order (include/fba.h, fba_pair_slots), by plain loops:
+    pair (m, J, e) = (pairs of all list rows before (m, J)) + e; returns (pair_base [M*nK + 1] with the total last,
+    q_slot [M, nQ, nK] = number of the pair (I, q_idx[m, I, e]), -1 beyond q_cnt)."""
+    M, nK = k_cnt.shape
+    nQ = q_cnt.shape[1]
+    pair_base = np.zeros((M * nK + 1,), np.int32)
+    number = {}
+    n = 0
+    for m in range(M):
+        for J in range(nK):
+            pair_base[m * nK + J] = n
+            for e in range(int(k_cnt[m, J])):
+                number[(m, int(k_idx[m, J, e]), J)] = n
+                n += 1
+    pair_base[M * nK] = n
+    q_slot = np.full((M, nQ, nK), -1, np.int32)
+    for m in range(M):
+        for I in range(nQ):
+            for e in range(int(q_cnt[m, I])):
+                q_slot[m, I, e] = number[(m, I, int(q_idx[m, I, e]))]
+    return pair_base, q_slot
+
+
 def tile_lists(block_mask, q_block, kv_block):
     """Brute-force tile lists (include/fba.h, fba_tile_lists) of a bool mask [nQ, nK] or [B, H, nQ, nK]: for every
     128-row query tile the key blocks selected by any of its eight 16-row groups, with one predicate bit per group; for

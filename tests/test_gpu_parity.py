@@ -365,7 +365,7 @@ def test_deterministic(gpu):
         assert torch.equal(a, b)
 
 
-def _full_size_properties(gpu, q, k, v, do, qbs, kbs, mask, check_permutation=True):
+def _full_size_properties(gpu, q, k, v, do, qbs, kbs, mask, check_permutation=True, hand_over=None):
     """Properties that need no oracle and hold at any size:
       * V = 1 gives O = 1 (softmax rows sum to one, also across lazily rescaled slabs);
       * doubling dO doubles dQ, dK, dV bit for bit (everything downstream of dO is linear; scaling by 2 is exact);
@@ -380,8 +380,8 @@ def _full_size_properties(gpu, q, k, v, do, qbs, kbs, mask, check_permutation=Tr
     del o1
     o, lse = fba.forward_with_lists(q, k, v, qbs, kbs, lists)
     assert torch.isfinite(o).all() and torch.isfinite(lse).all()
-    dq, dk, dv = fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists)
-    dq2, dk2, dv2 = fba.backward_with_lists(q, k, v, o, lse, do * 2, qbs, kbs, lists)
+    dq, dk, dv = fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists, hand_over=hand_over)
+    dq2, dk2, dv2 = fba.backward_with_lists(q, k, v, o, lse, do * 2, qbs, kbs, lists, hand_over=hand_over)
     for a, b in ((dq, dq2), (dk, dk2), (dv, dv2)):
         assert torch.isfinite(a).all() and torch.equal(a * 2, b)
     del dq2, dk2, dv2
@@ -418,7 +418,10 @@ def test_full_size_properties(gpu):
     B, H, S, bs, nb = 1, 24, 30720, 384, 80
     q, k, v, do = _full_size_inputs(gpu, B, H, S, 11)
     m = masks.random_block_mask(B, H, nb, nb, 32, 12).to(gpu)
-    _full_size_properties(gpu, q, k, v, do, bs, bs, m)
+    a = _full_size_properties(gpu, q, k, v, do, bs, bs, m, hand_over=True)
+    b = _full_size_properties(gpu, q, k, v, do, bs, bs, m, check_permutation=False, hand_over=False)
+    assert torch.equal(a[3], b[3]) and torch.equal(a[4], b[4])  # dK, dV: same kernel arithmetic on either path
+    assert (a[2].float() - b[2].float()).abs().max().item() <= 2e-2
 
 
 def test_full_attention_full_size_properties(gpu):
@@ -481,6 +484,68 @@ def test_asymmetric_full_size_properties(gpu):
     diag = torch.arange(nQ, device=gpu) * qbs // kbs
     assert m[0, :, torch.arange(nQ, device=gpu), diag].all()
     _full_size_properties(gpu, q, k, v, do, qbs, kbs, m)
+
+
+def test_pair_numbering_bit_exact(oracle, gpu):
+    """fba_pair_slots against the oracle's loop restatement: 2-D and per-(b,h) masks, empty rows and columns, the
+    benchmark's 80x80 masks."""
+    import flex_block_attn_amd as fba
+    from flex_block_attn_amd import masks
+
+    cases = [masks.bernoulli_block_mask(4, 4, 0.5, 0), masks.bernoulli_block_mask(65, 129, 0.5, 4), torch.zeros((7, 9), dtype=torch.bool),
+             torch.ones((30, 30), dtype=torch.bool), masks.random_block_mask(1, 24, 80, 80, 32, 5), masks.random_block_mask(2, 3, 17, 70, 5, 6),
+             masks.sta_3d_block_mask((5, 6, 10), (3, 3, 3)), torch.rand((1, 24, 540, 180), generator=torch.Generator().manual_seed(1)) < 0.1]
+    for m in cases:
+        lists = fba.compact_block_mask(m.to(gpu))
+        lists = fba.number_pairs(lists)
+        pair_base, q_slot, listed = lists.pair_base, lists.q_slot, lists.listed_pairs()
+        want_base, want_slot = oracle.pair_numbering(*oracle.compact_lists(m))
+        assert pair_base.dtype == torch.int32 and q_slot.dtype == torch.int32 and listed == int(m.sum())
+        assert np.array_equal(pair_base.cpu().numpy(), want_base), tuple(m.shape)
+        assert np.array_equal(q_slot.cpu().numpy(), want_slot), tuple(m.shape)
+
+
+BACKWARD_PATH_CASES = [
+    # B, Hq, Hkv, Sq, Skv, q_block, kv_block, mask dims, density
+    (1, 2, 2, 1536, 1536, 384, 384, 4, 0.5),
+    (1, 3, 3, 768, 768, 128, 128, 2, 0.6),     # one 2-D mask for three heads: per-head offset into the workspace
+    (2, 4, 2, 512, 1024, 128, 256, 4, 0.5),    # grouped kv heads, cross lengths, kv block larger than the q block
+    (1, 2, 1, 1024, 768, 256, 128, 4, 0.4),    # q block larger than the kv block
+    (1, 6, 2, 768, 1152, 384, 128, 2, 0.7),
+    (2, 2, 2, 384, 384, 128, 384, 4, 1.0),
+]
+
+
+@pytest.mark.parametrize("hand_over", [False, True], ids=["recompute", "handover"])
+@pytest.mark.parametrize("cfg", BACKWARD_PATH_CASES, ids=lambda c: "B%d_Hq%d_Hkv%d_Sq%d_Skv%d_q%d_k%d_m%d_p%s" % c)
+def test_both_backward_paths_against_oracle(oracle, gpu, cfg, hand_over):
+    """fba_bwd (dQ recomputes S and dP) and fba_bwd_handover (dQ from the dS the key-major kernel stored), each against
+    the C oracle; masks with an empty query block and an unselected key block."""
+    import flex_block_attn_amd as fba
+
+    B, Hq, Hkv, Sq, Skv, qbs, kbs, mdim, density = cfg
+    nQ, nK = Sq // qbs, Skv // kbs
+    g = torch.Generator().manual_seed(Sq + Skv + qbs)
+    m = torch.rand((nQ, nK) if mdim == 2 else (B, Hq, nQ, nK), generator=g) < density
+    if density < 1.0 and nQ > 1 and nK > 1:
+        m[..., 0, :] = False
+        m[..., :, nK - 1] = False
+        m[..., nQ - 1, 0] = True
+    q, k, v, do = oracle.seeded_qkv(B, Hq, Hkv, Sq, Skv, seed=Sq + kbs)
+    qb, kb, vb, dob = (t.to(torch.bfloat16) for t in (q, k, v, do))
+    o_ref, lse_ref = oracle.c_attention_forward(qb, kb, vb, m, qbs, kbs)
+    g_ref = oracle.c_attention_backward(qb, kb, vb, o_ref, lse_ref, dob, m, qbs, kbs)
+    qg, kg, vg, dog = (t.to(gpu) for t in (qb, kb, vb, dob))
+    lists = fba.compact_block_mask(m.to(gpu))
+    o, lse = fba.forward_with_lists(qg, kg, vg, qbs, kbs, lists)
+    print(f"backward path hand_over={hand_over} cfg={cfg}", flush=True)
+    grads = fba.backward_with_lists(qg, kg, vg, o, lse, dog, qbs, kbs, lists, hand_over=hand_over)
+    res = {}
+    for n, got, want in zip(("dq", "dk", "dv"), grads, g_ref):
+        _check(oracle, got, want, n, res)
+    other = fba.backward_with_lists(qg, kg, vg, o, lse, dog, qbs, kbs, lists, hand_over=not hand_over)
+    assert torch.equal(grads[1], other[1]) and torch.equal(grads[2], other[2])  # dK, dV do not depend on the path
+    assert (grads[0].float() - other[0].float()).abs().max().item() <= 2e-2
 
 
 def test_backward_statistics_against_oracle(oracle, gpu):

@@ -296,6 +296,32 @@ def test_tile_order_is_the_einops_rearrangement(oracle):
     assert torch.equal(x[idx], want) and sorted(idx.tolist()) == list(range(96))
 
 
+def test_pair_numbering(oracle):
+    """oracle.pair_numbering: the numbers are 0..n-1 in key-major list order (checked against numpy's cumsum and against
+    the lists themselves), and the query-major table points back at the same pair."""
+    for shape, p, seed in (((5, 7), 0.5, 0), ((2, 3, 6, 4), 0.4, 1), ((3, 3), 0.0, 2), ((1, 2, 4, 4), 1.0, 3)):
+        m = torch.rand(shape, generator=torch.Generator().manual_seed(seed)) < p
+        q_cnt, q_idx, k_cnt, k_idx = oracle.compact_lists(m)
+        pair_base, q_slot = oracle.pair_numbering(q_cnt, q_idx, k_cnt, k_idx)
+        M, nK = k_cnt.shape
+        nQ = q_cnt.shape[1]
+        assert np.array_equal(pair_base, np.concatenate([[0], np.cumsum(k_cnt.reshape(-1))]).astype(np.int32))
+        assert pair_base[-1] == int(m.sum())
+        seen = []
+        for mm in range(M):
+            for I in range(nQ):
+                for e in range(nK):
+                    n = q_slot[mm, I, e]
+                    if e >= q_cnt[mm, I]:
+                        assert n == -1
+                        continue
+                    J = q_idx[mm, I, e]
+                    pos = n - pair_base[mm * nK + J]
+                    assert 0 <= pos < k_cnt[mm, J] and k_idx[mm, J, pos] == I
+                    seen.append(int(n))
+        assert sorted(seen) == list(range(int(m.sum())))
+
+
 def test_sliding_tile_mask_restatement(oracle):
     """Pins oracle.sta_window / sta_3d_mask / sta_token_mask: hand-computed windows, a hand-listed row of an asymmetric
     grid, the Kronecker product of 1-D band matrices (numpy's kron fixes the T-major, W-minor enumeration: swapping two

@@ -19,7 +19,7 @@ def _case(gpu, B, H, Hkv, S, bs, keep, seed):
     nb = S // bs
     lists = fba.compact_block_mask(masks.random_block_mask(B, H, nb, nb, keep, seed).to(gpu))
     o, lse = fba.forward_with_lists(q, k, v, bs, bs, lists)
-    want = fba.backward_with_lists(q, k, v, o, lse, do, bs, bs, lists)  # fba_bwd with a torch-allocated stats buffer
+    want = fba.backward_with_lists(q, k, v, o, lse, do, bs, bs, lists, hand_over=False)  # fba_bwd with a torch-allocated stats buffer
     got = tuple(torch.full_like(t, float("nan")) for t in (q, k, v))
     torch.cuda.synchronize()
     before = torch.cuda.memory_allocated()
