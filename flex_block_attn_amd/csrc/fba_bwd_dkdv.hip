@@ -267,7 +267,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
 
     const int npairs = (nslabs + 1) >> 1;
     auto step = [&](auto half_c, int s2) {
-      if (2 * s2 + par < nslabs) compute(half_c);
+      // tile lists: a wave whose 32 keys are selected by neither half of the slab leaves the slab out (wave-uniform)
+      if (2 * s2 + par < nslabs && (!kTiled || ((bits_cmp >> (2 * kg)) & 3) != 0)) compute(half_c);
       if constexpr (kTiled) { next_bits(); next_bits(); }
       if constexpr (kHandOver) ho_advance(2);
       // this wave's copies of the next pair, requested one step ago, must have landed.  The two dS stores of this step are

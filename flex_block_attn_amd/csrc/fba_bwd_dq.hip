@@ -57,6 +57,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   const ConstIdx idx = const_idx(p.q_idx + mrow * p.nK);
   auto key_block = [&](int e) -> int { return kTiled ? idx[e] >> 8 : idx[e]; };
   const int group_bit = 1 << (2 * wave + (l32 >> 4));  // this lane's 16-row group in a tile-list entry
+  const int wave_bits = 3 << (2 * wave);               // both groups of this wave
   const int nsub = p.k_block / kSlab;
   const int nsteps = cnt * nsub;
 
@@ -131,14 +132,30 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     auto step = [&](auto ring_c, int t) {
       constexpr int R = decltype(ring_c)::value;
       const bool active = !kTiled || (bits_cmp & group_bit) != 0;
-      f32x16 s_cur, dp_cur;
-      scores(smem + R * kPairBytes, s_cur, dp_cur);
-      bf16x8 dsk[2];
+      // a wave whose two 16-row groups are both switched off for this slab has nothing to add (wave-uniform branch)
+      if (!kTiled || (bits_cmp & wave_bits) != 0) {
+        f32x16 s_cur, dp_cur;
+        scores(smem + R * kPairBytes, s_cur, dp_cur);
+        bf16x8 dsk[2];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        float pv = fast_exp2(__builtin_fmaf(s_cur[r], c, -lse2));
-        if constexpr (kTiled) pv = active ? pv : 0.f;  // a select, so that inf or NaN of a masked row is discarded
-        s_cur[r] = pv * (dp_cur[r] - dlt);
+        for (int r = 0; r < 16; ++r) {
+          float pv = fast_exp2(__builtin_fmaf(s_cur[r], c, -lse2));
+          if constexpr (kTiled) pv = active ? pv : 0.f;  // a select, so that inf or NaN of a masked row is discarded
+          s_cur[r] = pv * (dp_cur[r] - dlt);
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          dsk[j] = pack8(s_cur[8 * j + 0], s_cur[8 * j + 1], s_cur[8 * j + 2], s_cur[8 * j + 3], s_cur[8 * j + 4],
+                         s_cur[8 * j + 5], s_cur[8 * j + 6], s_cur[8 * j + 7]);
+        const char* k_t = smem + R * kPairBytes;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int mb = 0; mb < 4; ++mb) {
+            const int roff = 16 * j * kRowBytes;
+            const bf16x8 a = cat(lds_read_tr(k_t, tr.rd[mb][0] + roff), lds_read_tr(k_t, tr.rd[mb][1] + roff));
+            acc[mb] = mfma32(a, dsk[j], acc[mb]);
+          }
       }
       if constexpr (kTiled) {
         if (--rem_cmp == 0) {
@@ -147,19 +164,6 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
           bits_cmp = e_cmp < cnt ? idx[e_cmp] & 255 : 0;
         }
       }
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-        dsk[j] = pack8(s_cur[8 * j + 0], s_cur[8 * j + 1], s_cur[8 * j + 2], s_cur[8 * j + 3], s_cur[8 * j + 4],
-                       s_cur[8 * j + 5], s_cur[8 * j + 6], s_cur[8 * j + 7]);
-      const char* k_t = smem + R * kPairBytes;
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int mb = 0; mb < 4; ++mb) {
-          const int roff = 16 * j * kRowBytes;
-          const bf16x8 a = cat(lds_read_tr(k_t, tr.rd[mb][0] + roff), lds_read_tr(k_t, tr.rd[mb][1] + roff));
-          acc[mb] = mfma32(a, dsk[j], acc[mb]);
-        }
       // slab t+2 must have landed (first read in step t+1); the four copies of slab t+3 may still fly
       if (t + 3 < nsteps) wait_vmem<4>(); else wait_vmem<0>();
       __syncthreads();

@@ -213,22 +213,35 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     // predicate of the slab whose softmax is next (tile lists): all 16-row groups share the entry, each lane tests its bit
     int e_cmp = 0, rem_cmp = nsub;
     int bits_cmp = kTiled ? idx[0] & 255 : 255;
+    int bits_ahead = kTiled && cnt > 1 ? idx[1] & 255 : 0;  // predicate bits of the following list entry
+    // A wave whose two 16-row groups are both switched off for a slab leaves that slab's matrix work out altogether
+    // (wave-uniform branches); rows switched off inside an active wave are dealt with by selects.
+    const int wave_bits = 3 << (2 * wave);
+    bool w_prev = false;  // did this wave form P for the previous slab?
 
     // step t (t % 4 == R): O += P_{t-1} V_{t-1} | softmax(S_t) | S_{t+1} = K_{t+1} Q^T
     auto step = [&](auto ring_c, auto first_c, int t) {
       constexpr int R = decltype(ring_c)::value;
       constexpr bool kFirst = decltype(first_c)::value;
+      const bool w_cur = !kTiled || (bits_cmp & wave_bits) != 0;
+      const bool w_nxt = !kTiled || ((rem_cmp > 1 ? bits_cmp : bits_ahead) & wave_bits) != 0;
       // P_{t-1} was formed against the reference m of step t-1, so it must reach O before step t may raise m
-      if constexpr (!kFirst) pv_half(st, v_lds + ((R + 3) & 3) * kSlabBytes, p_prev);
+      if constexpr (!kFirst) {
+        if (w_prev) pv_half(st, v_lds + ((R + 3) & 3) * kSlabBytes, p_prev);
+      }
       const bool active = !kTiled || (bits_cmp & group_bit) != 0;
-      softmax_reference(st, s_cur, active);
-      const f32x16 s_nxt = qk_half(st, k_lds + ((R + 1) & 3) * kSlabBytes);  // past the last slab: stale data, unused
-      softmax_exp<kTiled>(st, s_cur, p_prev, active);  // p_prev := P_t
+      if (w_cur) softmax_reference(st, s_cur, active);
+      f32x16 s_nxt;
+      if (w_nxt) s_nxt = qk_half(st, k_lds + ((R + 1) & 3) * kSlabBytes);  // past the last slab: stale data, unused
+      else s_nxt = s_cur;
+      if (w_cur) softmax_exp<kTiled>(st, s_cur, p_prev, active);  // p_prev := P_t
+      w_prev = w_cur;
       if constexpr (kTiled) {
         if (--rem_cmp == 0) {
           rem_cmp = nsub;
           ++e_cmp;
-          bits_cmp = e_cmp < cnt ? idx[e_cmp] & 255 : 0;
+          bits_cmp = bits_ahead;
+          bits_ahead = e_cmp + 1 < cnt ? idx[e_cmp + 1] & 255 : 0;
         }
       }
       // P_t is only consumed after the barrier; without the pins its arithmetic sinks there, away from the MFMAs it is
@@ -257,7 +270,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
       step(IC<1>{}, std::false_type{}, t + 3);
     }
     // O += P_{n-1} V_{n-1}
-    pv_half(st, v_lds + ((nsteps - 1) & 3) * kSlabBytes, p_prev);
+    if (w_prev) pv_half(st, v_lds + ((nsteps - 1) & 3) * kSlabBytes, p_prev);
   }
 
   // epilogue: O = O^T / l, LSE = ln2 * (c m + log2 l)
