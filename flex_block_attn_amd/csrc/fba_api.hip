@@ -355,7 +355,7 @@ int32_t fba_bwd_handover(const void* q, const void* k, const void* v, const void
 
 namespace {
 
-// Workspace of fba_bwd_noalloc: the two statistics planes of backward (lse * log2(e), delta) for up to kScratchRows
+// Workspace of fba_bwd_noalloc: the two statistics planes of backward (lse * log2(e), -delta) for up to kScratchRows
 // query rows, 32 MiB, held by every GPU the library is loaded on until the process ends.  In host code the array's name
 // is only a handle for hipGetSymbolAddress; kernels get the device address looked up below.
 constexpr int64_t kScratchRows = 1LL << 22;

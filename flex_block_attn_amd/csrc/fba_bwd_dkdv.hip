@@ -9,12 +9,13 @@
 // Work-group = 128 key rows of one (batch, kv head), eight waves, two per SIMD.  Wave w works on keys 32 (w % 4) ..+31
 // and on every second 32-query slab of the list (w / 4 = parity of the slab), lane = key:
 //   S = Q K^T, dP = dO V^T             A = Q / dO slab rows, B = K / V rows, all from LDS (128-bit fetches)
-//   P = exp2(c S - lse2[q]),  dS = P o (dP - delta[q])          (lse2, delta per accumulator row, read from LDS)
+//   P = exp2(c S - lse2[q]),  dS = P o (dP - delta[q])          (lse2, -delta per accumulator row, read from LDS; the dP
+//                                                               accumulators start from -delta)
 //   dV^T += dO^T P,  dK^T += Q^T dS    A = dO / Q slab through transposing LDS fetches, B = P / dS packed to bf16
 // The two waves of a key group hold partial sums over their slabs; at the end they swap halves through LDS (one sends
 // its dV part and finishes dK, the other the reverse).  Two waves per SIMD keep the matrix pipe busy while one of them
 // waits for LDS or runs the softmax; that is why K and V stay in LDS instead of 64 registers per lane.
-// LDS: ring of four (Q slab | dO slab | lse2 | delta) buffers = two slab pairs (while one pair is being worked on, the
+// LDS: ring of four (Q slab | dO slab | lse2 | -delta) buffers = two slab pairs (while one pair is being worked on, the
 // other is in flight global -> LDS), then the K tile and the V tile (32 KiB each).
 #include <type_traits>
 
@@ -27,7 +28,7 @@ namespace {
 
 constexpr int kSlab = 32;
 constexpr int kSlabBytes = kSlab * kRowBytes;       // 8 KiB
-constexpr int kStatBytes = 2 * kSlab * 4;           // lse2[32] | delta[32]
+constexpr int kStatBytes = 2 * kSlab * 4;           // lse2[32] | -delta[32]
 constexpr int kStageBytes = 2 * kSlabBytes + kStatBytes;
 constexpr int kRing = 4;
 constexpr int kTileBytes = 128 * kRowBytes;         // K or V tile, 32 KiB
@@ -83,7 +84,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
   const uint32_t lds0 = lds_addr(smem);
   const uint32_t ring_dst = lds0 + kRingBase;
   const int64_t rows_total = (int64_t)p.B * p.Hq * p.Sq;
-  // statistics copy: lanes 0..31 fetch lse2[row0 + l], lanes 32..63 fetch delta[row0 + l - 32]
+  // statistics copy: lanes 0..31 fetch lse2[row0 + l], lanes 32..63 fetch -delta[row0 + l - 32]
   const uint32_t stat_off = (uint32_t)((lane >> 5) * rows_total * 4 + (lane & 31) * 4);
   const float c = p.scale_log2e;
 
@@ -217,8 +218,13 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     auto compute = [&](auto half_c) {
       constexpr int so = decltype(half_c)::value * 2 * kStageBytes;  // buffers 0, 1 or 2, 3
       f32x16 s, dp;
+      // accumulator element 4g + e of half-wave h is query row 8g + 4h + e of the slab; dP starts from -delta of its row
 #pragma unroll
-      for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 d4 = *reinterpret_cast<const f32x4*>(smem + so + st_off + 4 * kSlab + 32 * g);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { s[4 * g + e] = 0.f; dp[4 * g + e] = d4[e]; }
+      }
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
         s = mfma32(lds_read_b128(smem + so, q_off[ks]), lds_read_b128(smem, k_off[ks]), s);
@@ -228,15 +234,14 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
       const bool on0 = !kTiled || ((bits_cmp >> (2 * kg)) & 1) != 0;
       const bool on1 = !kTiled || ((bits_cmp >> (2 * kg + 1)) & 1) != 0;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {  // accumulator element 4g + e of half-wave h is query row 8g + 4h + e of the slab
+      for (int g = 0; g < 4; ++g) {
         const f32x4 l4 = *reinterpret_cast<const f32x4*>(smem + so + st_off + 32 * g);
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(smem + so + st_off + 4 * kSlab + 32 * g);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           float pv = fast_exp2(__builtin_fmaf(s[4 * g + e], c, -l4[e]));
           if constexpr (kTiled) pv = (g < 2 ? on0 : on1) ? pv : 0.f;  // a select: inf or NaN of a masked row is discarded
           s[4 * g + e] = pv;
-          dp[4 * g + e] = pv * (dp[4 * g + e] - d4[e]);
+          dp[4 * g + e] = pv * dp[4 * g + e];
         }
       }
       bf16x8 pk[2], dsk[2];

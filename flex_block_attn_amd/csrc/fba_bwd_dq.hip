@@ -70,7 +70,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   }
   const int64_t rows_total = (int64_t)p.B * p.Hq * p.Sq;
   const float lse2 = p.stats[qrow0 + l32];
-  const float dlt = p.stats[rows_total + qrow0 + l32];
+  const float neg_dlt = p.stats[rows_total + qrow0 + l32];  // -delta of this lane's row
   const float c = p.scale_log2e;
 
   RowMajorOffsets rm;
@@ -141,7 +141,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
         for (int r = 0; r < 16; ++r) {
           float pv = fast_exp2(__builtin_fmaf(s_cur[r], c, -lse2));
           if constexpr (kTiled) pv = active ? pv : 0.f;  // a select, so that inf or NaN of a masked row is discarded
-          s_cur[r] = pv * (dp_cur[r] - dlt);
+          s_cur[r] = pv * (dp_cur[r] + neg_dlt);
         }
 #pragma unroll
         for (int j = 0; j < 2; ++j)

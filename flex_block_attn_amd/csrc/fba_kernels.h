@@ -33,7 +33,7 @@ struct BwdParams {
   const __bf16* k;
   const __bf16* v;
   const __bf16* d_o;
-  const float* stats;  // [2, B, Hq, Sq]: lse * log2(e), then delta = rowsum(dO o O)
+  const float* stats;  // [2, B, Hq, Sq]: lse * log2(e), then -delta = -rowsum(dO o O)
   __bf16* dq;
   __bf16* dk;
   __bf16* dv;

@@ -185,9 +185,11 @@ hipError_t launch_pair_slots(const int32_t* q_cnt, const int32_t* q_idx, const i
   return hipGetLastError();
 }
 
-// Backward statistics, one pass over O and dO: stats[r] = lse[r] * log2(e) and stats[rows + r] = delta[r] =
-// sum_c dO[r, c] * O[r, c] in fp32 (reference: bwd_attend_prep_ker, flex_block_attn_h100.cu:375-379).  The backward
-// kernels exponentiate in base 2, hence the pre-scaled LSE.  16 lanes per row (16 bytes of each operand per lane).
+// Backward statistics, one pass over O and dO: stats[r] = lse[r] * log2(e) and stats[rows + r] = -delta[r] =
+// -sum_c dO[r, c] * O[r, c] in fp32 (reference: bwd_attend_prep_ker, flex_block_attn_h100.cu:375-379).  The backward
+// kernels exponentiate in base 2, hence the pre-scaled LSE; they start the dP accumulators from the second plane, so that
+// the matrix instructions themselves form dP - delta (the reference preloads its accumulator the same way,
+// flex_block_attn_h100.cu:445-467), hence the sign.  16 lanes per row (16 bytes of each operand per lane).
 __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void bwd_stats_kernel(const __bf16* __restrict__ o,
                                                                                         const __bf16* __restrict__ d_o,
                                                                                         const float* __restrict__ lse,
@@ -205,7 +207,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void bwd_stats
     acc += __shfl_xor(acc, 1);
     if (sub == 0) {
       stats[r] = lse[r] * 1.4426950408889634f;
-      stats[rows + r] = acc;
+      stats[rows + r] = -acc;
     }
   }
 }

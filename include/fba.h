@@ -66,7 +66,7 @@ int32_t fba_fwd(const void* q, const void* k, const void* v, void* o, float* lse
 /*
  * Backward, three stream-ordered launches.  Replaces attn_backward (attn.cpp:30,
  * flex_block_attn_h100.cu:1009-1267): bwd_attend_prep_ker (:324-389) and bwd_attend_ker (:572-802).
- *   stats    [2, B, Hq, Sq] fp32 workspace written by the call: lse * log2(e), then delta = rowsum(dO o O)
+ *   stats    [2, B, Hq, Sq] fp32 workspace written by the call: lse * log2(e), then -delta = -rowsum(dO o O)
  *   dq       [B, Hq, Sq, 128] bf16;  dk, dv [B, Hkv, Skv, 128] bf16 (summed over the query heads of a GQA group)
  * Every output element is written exactly once; no buffer needs clearing beforehand.
  */

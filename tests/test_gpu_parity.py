@@ -549,7 +549,7 @@ def test_both_backward_paths_against_oracle(oracle, gpu, cfg, hand_over):
 
 
 def test_backward_statistics_against_oracle(oracle, gpu):
-    """fba_bwd_stats alone: stats[0] = lse * log2(e), stats[1] = delta = rowsum(dO o O), against the C oracle's
+    """fba_bwd_stats alone: stats[0] = lse * log2(e), stats[1] = -delta = -rowsum(dO o O), against the C oracle's
     oracle_bwd_delta (flex_block_attn_h100.cu:375-379) on the same bf16 values; rows that are not a multiple of the
     kernel's 16-row groups included."""
     import ctypes
@@ -570,7 +570,7 @@ def test_backward_statistics_against_oracle(oracle, gpu):
         stats = torch.full((2, rows), float("nan"), dtype=torch.float32, device=gpu)
         _lib.call("fba_bwd_stats", _ptr(og), _ptr(dg), _ptr(lg), _ptr(stats), rows, 128, _stream())
         got = stats.cpu()
-        assert (got[1] - torch.from_numpy(want)).abs().max().item() <= 1e-4  # fp32 sums of 128 products of N(0,1) pairs
+        assert (-got[1] - torch.from_numpy(want)).abs().max().item() <= 1e-4  # fp32 sums of 128 products of N(0,1) pairs
         want_l2 = lse.double() * 1.4426950408889634
         assert got[0, 0].item() == float("-inf")
         if rows > 1:
