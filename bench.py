@@ -144,6 +144,27 @@ def cpu_baseline(seconds_budget=12.0):
     }
 
 
+def probe_atomics():
+    """fp32 atomic adds of 512-byte rows (one query row of dQ) at random rows of a [24 * 30720, 128] fp32 buffer, through
+    torch's index_add_ (a gather of src rows + one hardware atomic add per element), against a plain copy of the same bytes.
+    The reference's backward adds its dQ partials this way (flex_block_attn_h100.cu:707-708); with 128-key tiles that is
+    36 GB of adds per launch of the default workload."""
+    dev = torch.device("cuda:0")
+    rows, n = 24 * 30720, 4 * 1024 * 1024
+    g = torch.Generator(device="cpu").manual_seed(0)
+    dst = torch.zeros((rows, D), dtype=torch.float32, device=dev)
+    src = torch.randn((n, D), generator=g, dtype=torch.float32).to(dev)
+    idx = torch.randint(0, rows, (n,), generator=g).to(dev)
+    out = torch.empty_like(src)
+    add_ms = statistics.median(time_events(lambda: dst.index_add_(0, idx, src), 2, 5))
+    copy_ms = statistics.median(time_events(lambda: out.copy_(src), 2, 5))
+    nbytes = src.numel() * 4
+    res = {"probe": "fp32 atomic adds, 512-byte rows at random rows of a 377 MB buffer (torch index_add_)", "bytes_added": nbytes,
+           "atomic_add_ms": add_ms, "atomic_add_GB/s": nbytes / add_ms * 1e-6, "plain_copy_ms": copy_ms, "plain_copy_GB/s": nbytes / copy_ms * 1e-6,
+           "dq_partial_bytes_per_launch_128_key_tiles": 4.0 * 61440 * 384 * 128 * 3, "dq_partial_bytes_per_launch_384_key_owner": 4.0 * 61440 * 384 * 128}
+    print(json.dumps(res), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -156,7 +177,12 @@ def main():
                     help="zeros: all-zero q, k, v, dO (a probe of the power limit, not a benchmark figure)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy three times, as the known-size yardstick for rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--probe-atomics", action="store_true",
+                    help="instead of the benchmark, measure the throughput of fp32 atomic adds into a dQ-sized buffer (what a fused "
+                         "backward with reducing stores, as in the reference, would be bound by) and print it")
     args = ap.parse_args()
+    if args.probe_atomics:
+        return probe_atomics()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU only: every box in this build has a single MI355X (use --gpus 1)")
     if not torch.cuda.is_available():
