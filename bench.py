@@ -206,7 +206,7 @@ def main():
     mask_fn = w["mask_fn"]
 
     def step():
-        lists = fba.compact_block_mask(mask_fn() if mask_fn else mask)
+        lists = fba.compact_block_mask(mask_fn() if mask_fn else mask, with_pair_numbers=not args.recompute)
         o, lse = fba.forward_with_lists(q, k, v, qbs, kbs, lists)
         return fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists, hand_over=False if args.recompute else None)
 

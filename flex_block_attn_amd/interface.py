@@ -74,8 +74,9 @@ def _require_device(t, name):
         raise ValueError(f"{name} must be a GPU tensor (the HIP kernels have no CPU fallback)")
 
 
-def compact_block_mask(block_mask):
-    """bool block mask [nQ, nK] or [B, H, nQ, nK] (GPU) -> BlockLists, via the compaction kernel."""
+def compact_block_mask(block_mask, with_pair_numbers=False):
+    """bool block mask [nQ, nK] or [B, H, nQ, nK] (GPU) -> BlockLists, via the compaction kernel.  `with_pair_numbers`
+    also numbers the pairs right away (what the dS hand-over of backward needs; see `number_pairs`)."""
     if block_mask.dtype != torch.bool:
         raise TypeError(f"block_mask must be a bool tensor, got {block_mask.dtype}")
     if block_mask.dim() not in (2, 4):
@@ -91,9 +92,10 @@ def compact_block_mask(block_mask):
     k_idx = torch.empty((mask_bh, nK, nQ), dtype=torch.int32, device=dev)
     with torch.cuda.device(dev):
         _lib.call("fba_mask_compact", _ptr(m), mask_bh, nQ, nK, _ptr(q_cnt), _ptr(q_idx), _ptr(k_cnt), _ptr(k_idx), _stream())
-    # numbered right away: the host copy of the pair count is then ordered before whatever the caller enqueues next, and
-    # backward finds it without waiting for the forward kernel
-    return number_pairs(BlockLists(q_cnt, q_idx, k_cnt, k_idx, mask_bh, nQ, nK))
+    lists = BlockLists(q_cnt, q_idx, k_cnt, k_idx, mask_bh, nQ, nK)
+    # numbered right away when a backward pass will follow: the host copy of the pair count is then ordered before
+    # whatever the caller enqueues next, and backward finds it without waiting for the forward kernel
+    return number_pairs(lists) if with_pair_numbers else lists
 
 
 def needs_tile_lists(q_block_size, kv_block_size):
@@ -125,11 +127,11 @@ def tile_block_mask(block_mask, q_block_size, kv_block_size):
     return BlockLists(qt_cnt, qt_ent, kt_cnt, kt_ent, mask_bh, nQ, nK, tiled=True)
 
 
-def lists_for(block_mask, q_block_size, kv_block_size):
+def lists_for(block_mask, q_block_size, kv_block_size, with_pair_numbers=False):
     """The list flavour the kernels need for these block sizes."""
     if needs_tile_lists(q_block_size, kv_block_size):
         return tile_block_mask(block_mask, q_block_size, kv_block_size)
-    return compact_block_mask(block_mask)
+    return compact_block_mask(block_mask, with_pair_numbers)
 
 
 def _check_qkv(q, k, v):
@@ -328,7 +330,7 @@ class FlexBlockAttnFunc(torch.autograd.Function):
     def forward(ctx, q, k, v, q_block_size, kv_block_size, block_mask, is_grad_enabled):
         _check_blocks(q, k, q_block_size, kv_block_size, block_mask)
         is_grad = is_grad_enabled and any(x.requires_grad for x in [q, k, v])
-        lists = lists_for(block_mask, q_block_size, kv_block_size)
+        lists = lists_for(block_mask, q_block_size, kv_block_size, with_pair_numbers=is_grad)
         o, lse = forward_with_lists(q, k, v, q_block_size, kv_block_size, lists)
         if is_grad:
             ctx.save_for_backward(q, k, v, o, lse)
