@@ -252,7 +252,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
       }
       if constexpr (kHandOver) {
         char* unit = reinterpret_cast<char*>(p.ds_ws) + (h_slot0 + h_e) * pair_bytes +
-                     (int64_t)((((h_s >> 2) * nsub_k + t_key) * 4 + (h_s & 3)) * kDsUnitBytes);
+                     ((int64_t)((h_s >> 2) * nsub_k + t_key) * 4 + (h_s & 3)) * kDsUnitBytes;
         // written once, read once by another kernel much later: streaming stores, so that they do not push the Q / dO
         // slabs that other work-groups are about to fetch out of L2
         __builtin_nontemporal_store(dsk[0], reinterpret_cast<bf16x8*>(unit + ho_off0));
