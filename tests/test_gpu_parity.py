@@ -548,6 +548,28 @@ def test_both_backward_paths_against_oracle(oracle, gpu, cfg, hand_over):
     assert (grads[0].float() - other[0].float()).abs().max().item() <= 2e-2
 
 
+def test_backward_falls_back_without_workspace(gpu, monkeypatch):
+    """With the workspace limit at zero the automatic choice is the recomputing backward: same bits as hand_over=False,
+    and no dS workspace is allocated."""
+    import flex_block_attn_amd as fba
+    from flex_block_attn_amd import interface, masks
+
+    g = torch.Generator(device="cpu").manual_seed(3)
+    q, k, v, do = (torch.randn((1, 2, 768, 128), generator=g).to(torch.bfloat16).to(gpu) for _ in range(4))
+    lists = fba.compact_block_mask(masks.bernoulli_block_mask(6, 6, 0.5, 1).to(gpu))
+    o, lse = fba.forward_with_lists(q, k, v, 128, 128, lists)
+    want = fba.backward_with_lists(q, k, v, o, lse, do, 128, 128, lists, hand_over=False)
+    monkeypatch.setattr(interface, "DS_WORKSPACE_LIMIT_GIB", 0.0)
+    got = fba.backward_with_lists(q, k, v, o, lse, do, 128, 128, lists)
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+    # an empty mask has no pair to hand over: both settings give zero gradients
+    empty = fba.compact_block_mask(torch.zeros((6, 6), dtype=torch.bool, device=gpu))
+    o0, lse0 = fba.forward_with_lists(q, k, v, 128, 128, empty)
+    for t in fba.backward_with_lists(q, k, v, o0, lse0, do, 128, 128, empty, hand_over=True):
+        assert t.abs().max().item() == 0.0
+
+
 def test_backward_statistics_against_oracle(oracle, gpu):
     """fba_bwd_stats alone: stats[0] = lse * log2(e), stats[1] = -delta = -rowsum(dO o O), against the C oracle's
     oracle_bwd_delta (flex_block_attn_h100.cu:375-379) on the same bf16 values; rows that are not a multiple of the
