@@ -144,6 +144,18 @@ def cpu_baseline(seconds_budget=12.0):
     }
 
 
+def sustained_mfma_tflops(dev, data):
+    """TFLOP/s of a register-only loop of v_mfma_f32_32x32x16_bf16 (fba_probe_mfma) on N(0,1) or all-zero operands."""
+    from flex_block_attn_amd import _lib
+    from flex_block_attn_amd.interface import _ptr, _stream
+
+    wgs, iters = 2048, 100000
+    src = torch.randn((1024,), generator=torch.Generator(device="cpu").manual_seed(7)).to(dev) if data == "normal" else None
+    sink = torch.empty((wgs * 256,), dtype=torch.float32, device=dev)
+    ms = statistics.median(time_events(lambda: _lib.call("fba_probe_mfma", _ptr(src) if src is not None else None, _ptr(sink), wgs, iters, _stream()), 1, 3))
+    return wgs * 4.0 * iters * 4 * 32768 / (ms * 1e-3) * 1e-12
+
+
 def probe_atomics():
     """fp32 atomic adds of 512-byte rows (one query row of dQ) at random rows of a [24 * 30720, 128] fp32 buffer, through
     torch's index_add_ (a gather of src rows + one hardware atomic add per element), against a plain copy of the same bytes.
@@ -277,6 +289,12 @@ def main():
     dominant = max(in_step, key=lambda n: kms[n]["mean_ms"])
     roofline = dict(rooflines[dominant])
     roofline["kernel"] = dominant
+    # what a bare MFMA loop sustains right now on this GPU, on N(0,1) operands and on zeros (the clock follows the data)
+    sustained = {d: sustained_mfma_tflops(dev, d) for d in ("normal", "zeros")}
+    log(f"bare MFMA loop: {sustained['normal']:.0f} TFLOP/s on N(0,1) operands, {sustained['zeros']:.0f} on zeros (nominal peak {PEAK_BF16_TFLOPS:.0f})")
+    if roofline["bound"] == "mfma":
+        roofline["sustained_peak"] = sustained["normal"]
+        roofline["frac_of_sustained"] = roofline["achieved"] / sustained["normal"]
 
     mask_bytes = mask.numel() + 4 * (2 * nnz // (1 if mask.dim() == 4 else B * H) + lists.mask_bh * (lists.nQ + lists.nK))
     compaction = {"ms": kms["mask_compact"]["mean_ms"], "algorithmic_bytes": mask_bytes, "GB/s": mask_bytes / (kms["mask_compact"]["mean_ms"] * 1e-3) * 1e-9, "peak_GB/s": PEAK_HBM_GBS}
@@ -291,6 +309,7 @@ def main():
         "frac_of_bf16_peak": value / PEAK_BF16_TFLOPS,
         "kernels_ms": {n: kms[n]["mean_ms"] for n in kms},
         "rooflines": rooflines,
+        "bare_mfma_loop_TFLOP/s": sustained,
         "mask_compaction": compaction,
     }
     if mask_fn:

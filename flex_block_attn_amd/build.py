@@ -15,7 +15,7 @@ import sys
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_NAME = "libfba_gfx950.so"
 LIB_PATH = os.path.join(CSRC, LIB_NAME)
-SOURCES = ["fba_api.hip", "fba_mask_compact.hip", "fba_ssta_mask.hip", "fba_fwd.hip", "fba_bwd_dq.hip", "fba_bwd_dq_ds.hip", "fba_bwd_dkdv.hip"]
+SOURCES = ["fba_api.hip", "fba_mask_compact.hip", "fba_ssta_mask.hip", "fba_fwd.hip", "fba_bwd_dq.hip", "fba_bwd_dq_ds.hip", "fba_bwd_dkdv.hip", "fba_probe.hip"]
 
 # Per-file extras.  --amdgpu-mfma-vgpr-form keeps MFMA accumulators in ordinary VGPRs, so the softmax arithmetic on
 # them needs no accumulator-register copies; it pays off where the whole working set fits 256 registers.

@@ -272,6 +272,13 @@ int32_t fba_bwd(const void* q, const void* k, const void* v, const void* o, cons
                   q_block, k_block, hip_stream, false);
 }
 
+int32_t fba_probe_mfma(const float* src, float* sink, int32_t work_groups, int32_t iters, void* hip_stream) {
+  if (work_groups <= 0 || iters <= 0) return fail(FBA_ERR_INVALID, "work_groups and iters must be positive (got %d %d)", work_groups, iters);
+  if (!sink) return fail(FBA_ERR_INVALID, "sink is null");
+  hipError_t e = fba::launch_probe_mfma(src, sink, work_groups, iters, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "probe launch");
+}
+
 int32_t fba_pair_slots(const int32_t* q_cnt, const int32_t* q_idx, const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh,
                        int32_t nQ, int32_t nK, int32_t* pair_base, int32_t* q_slot, void* hip_stream) {
   if (mask_bh <= 0 || nQ <= 0 || nK <= 0)

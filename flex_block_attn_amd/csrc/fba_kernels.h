@@ -75,6 +75,7 @@ hipError_t launch_bwd_stats(const __bf16* o, const __bf16* d_o, const float* lse
 hipError_t launch_bwd_dq(BwdParams p, hipStream_t stream);
 hipError_t launch_bwd_dkdv(BwdParams p, hipStream_t stream);
 hipError_t launch_bwd_dq_from_ds(BwdParams p, hipStream_t stream);
+hipError_t launch_probe_mfma(const float* src, float* sink, int work_groups, int iters, hipStream_t stream);
 hipError_t launch_pair_slots(const int32_t* q_cnt, const int32_t* q_idx, const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh,
                              int nQ, int nK, int32_t* pair_base, int32_t* q_slot, hipStream_t stream);
 

@@ -175,6 +175,15 @@ int32_t fba_ssta_mask(const float* q_mean, const float* k_mean, const uint8_t* b
 int32_t fba_tile_permute(const void* x, void* out, int64_t n_seq, int32_t T, int32_t H, int32_t W, int32_t tile_t,
                          int32_t tile_h, int32_t tile_w, int32_t head_dim, int32_t to_tiles, void* hip_stream);
 
+/*
+ * Diagnostic, no counterpart in the reference: `work_groups` x 4 waves each issue `iters` x 4 independent
+ * v_mfma_f32_32x32x16_bf16 on register operands taken from src (1024 floats in device memory; null: all-zero operands)
+ * and write a checksum per thread to sink (work_groups * 256 floats).  The launch executes
+ * work_groups * 4 * iters * 4 * 32768 FLOP; timed by the caller it gives the rate the matrix pipe sustains on such data,
+ * which on this GPU depends on the data (the clock follows the switching activity).
+ */
+int32_t fba_probe_mfma(const float* src, float* sink, int32_t work_groups, int32_t iters, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -614,3 +614,18 @@ def test_sweep_harness_runs(gpu, tmp_path):
             rows = list(csv.DictReader(open(tmp_path / f"{mode}_{kind}_results_384.csv")))
             assert len(rows) == 1 and list(rows[0].keys()) == lead + cols
             assert int(rows[0]["seq_len"]) == 768 and all(float(rows[0][c]) > 0 for c in cols)
+
+
+def test_matrix_pipe_probe(gpu):
+    """fba_probe_mfma: zero operands give zero checksums; with operands a[t], b[t] every accumulator element of a wave's
+    32x32 tile is a 16-term dot product repeated 4 * iters times, so the checksums are finite and scale with iters."""
+    from flex_block_attn_amd import _lib
+    from flex_block_attn_amd.interface import _ptr, _stream
+
+    sink = torch.full((4 * 256,), float("nan"), device=gpu)
+    _lib.call("fba_probe_mfma", None, _ptr(sink), 4, 10, _stream())
+    assert (sink == 0).all()
+    src = torch.full((1024,), 0.5, device=gpu)
+    _lib.call("fba_probe_mfma", _ptr(src), _ptr(sink), 4, 10, _stream())
+    # each MFMA adds 16 * 0.25 = 4 to every element; 10 of them per accumulator, 4 accumulators x 16 elements summed
+    assert torch.equal(sink, torch.full_like(sink, 4.0 * 10 * 64))
