@@ -196,7 +196,12 @@ def _check_lists(lists, q, B, Hq, Sq, Skv, q_block_size, kv_block_size):
         shapes = ((M, Sq // 128), (M, Sq // 128, lists.nK), (M, Skv // 128), (M, Skv // 128, Sq // 32))
     else:
         shapes = ((M, lists.nQ), (M, lists.nQ, lists.nK), (M, lists.nK), (M, lists.nK, lists.nQ))
-    for name, t, shape in zip(("q_cnt", "q_idx", "k_cnt", "k_idx"), (lists.q_cnt, lists.q_idx, lists.k_cnt, lists.k_idx), shapes):
+    names, tensors = ["q_cnt", "q_idx", "k_cnt", "k_idx"], [lists.q_cnt, lists.q_idx, lists.k_cnt, lists.k_idx]
+    if lists.pair_base is not None:
+        names += ["pair_base", "q_slot"]
+        tensors += [lists.pair_base, lists.q_slot]
+        shapes += ((M * lists.nK + 1,), (M, lists.nQ, lists.nK))
+    for name, t, shape in zip(names, tensors, shapes):
         if t.dtype != torch.int32 or t.device != q.device or not t.is_contiguous() or tuple(t.shape) != shape:
             raise ValueError(f"block lists: {name} must be a contiguous int32 tensor of shape {shape} on {q.device}, "
                              f"got {tuple(t.shape)} {t.dtype} on {t.device}")

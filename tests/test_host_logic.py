@@ -286,6 +286,12 @@ def test_block_lists_are_validated_before_any_launch():
         _check_lists(bad, q, 1, 2, 256, 256, 128, 128)
     with pytest.raises(ValueError, match="sequence lengths"):
         _check_lists(lists(), q, 1, 2, 512, 256, 128, 128)
+    numbered = lists()
+    numbered.pair_base, numbered.q_slot = torch.zeros((3,), **i32), torch.zeros((1, 2, 2), **i32)
+    _check_lists(numbered, q, 1, 2, 256, 256, 128, 128)
+    numbered.pair_base = torch.zeros((4,), **i32)
+    with pytest.raises(ValueError, match="pair_base"):
+        _check_lists(numbered, q, 1, 2, 256, 256, 128, 128)
     tiled = BlockLists(torch.zeros((1, 2), **i32), torch.zeros((1, 2, 4), **i32), torch.zeros((1, 2), **i32), torch.zeros((1, 2, 8), **i32), 1, 4, 4, tiled=True)
     _check_lists(tiled, q, 1, 2, 256, 256, 64, 64)
     tiled.k_idx = torch.zeros((1, 2, 4), **i32)
