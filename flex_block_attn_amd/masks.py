@@ -4,6 +4,7 @@ The first group keeps the names and argument order of the reference's caller-sid
 (benchmark/utils/utils.py:69-119) so that code written against them runs unchanged.  The second group builds the
 masks of the benchmark configurations directly as tensors (no Python loop over blocks).
 """
+import itertools
 import random
 
 import numpy as np
@@ -37,9 +38,11 @@ def create_sparse_mask(Q, block_size, selected_blocks):
     """(row, col) pairs -> bool [block_num, block_num] on Q's device (benchmark/utils/utils.py:94-103)."""
     block_num = int(Q.size(2) / block_size)
     m = np.zeros((block_num, block_num), dtype=bool)
-    if len(selected_blocks):
-        ij = np.asarray(selected_blocks, dtype=np.int64).reshape(-1, 2)
-        m[ij[:, 0], ij[:, 1]] = True
+    n = len(selected_blocks)
+    if n:
+        # flattening the pairs through an iterator is several times faster than np.asarray on a list of tuples
+        flat = np.fromiter(itertools.chain.from_iterable(selected_blocks), dtype=np.int64, count=2 * n)
+        m[flat[0::2], flat[1::2]] = True
     return torch.from_numpy(m).to(Q.device)
 
 
