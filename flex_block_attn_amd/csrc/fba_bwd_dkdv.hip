@@ -198,20 +198,21 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     wait_vmem<0>();
     __syncthreads();
 
-    // per-lane fetch offsets with the wave's share folded in: slab offsets carry the parity's buffer, tile offsets the key
-    // group's rows; what remains (pair, Q or dO, K or V, row group) is a compile-time immediate
-    int q_off[8], k_off[8], t_off[4][2];
+    // per-lane fetch addresses with the wave's share folded in: slab addresses carry the parity's buffer, tile addresses
+    // the key group's rows; what remains (pair, Q or dO, K or V, row group) is a compile-time displacement
+    const LdsPtr lds = lds_ptr(smem);
+    LdsPtr q_ptr[8], k_ptr[8], t_ptr[4][2];
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-      q_off[ks] = rm.rd[ks] + par * kStageBytes;
-      k_off[ks] = rm.rd[ks] + kTileBase + kg * kSlabBytes;
+      q_ptr[ks] = lds + rm.rd[ks] + par * kStageBytes;
+      k_ptr[ks] = lds + rm.rd[ks] + kTileBase + kg * kSlabBytes;
     }
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb) {
-      t_off[mb][0] = tr.rd[mb][0] + par * kStageBytes;
-      t_off[mb][1] = tr.rd[mb][1] + par * kStageBytes;
+      t_ptr[mb][0] = lds + tr.rd[mb][0] + par * kStageBytes;
+      t_ptr[mb][1] = lds + tr.rd[mb][1] + par * kStageBytes;
     }
-    const int st_off = par * kStageBytes + 2 * kSlabBytes + 16 * h;
+    const LdsPtr st_ptr = lds + par * kStageBytes + 2 * kSlabBytes + 16 * h;
 
     // One slab against this wave's 32 keys.  Operands are fetched right where they are used: with two waves per SIMD the
     // other wave's matrix instructions cover the wait (fetching a step ahead into a second register set measured slower).
@@ -221,21 +222,21 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
       // accumulator element 4g + e of half-wave h is query row 8g + 4h + e of the slab; dP starts from -delta of its row
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const f32x4 d4 = *reinterpret_cast<const f32x4*>(smem + so + st_off + 4 * kSlab + 32 * g);
+        const f32x4 d4 = lds_read_f32x4(st_ptr + so + 4 * kSlab + 32 * g);
 #pragma unroll
         for (int e = 0; e < 4; ++e) { s[4 * g + e] = 0.f; dp[4 * g + e] = d4[e]; }
       }
 #pragma unroll
       for (int ks = 0; ks < 8; ++ks) {
-        s = mfma32(lds_read_b128(smem + so, q_off[ks]), lds_read_b128(smem, k_off[ks]), s);
-        dp = mfma32(lds_read_b128(smem + so + kSlabBytes, q_off[ks]), lds_read_b128(smem + kTileBytes, k_off[ks]), dp);
+        s = mfma32(lds_read_b128(q_ptr[ks] + so), lds_read_b128(k_ptr[ks]), s);
+        dp = mfma32(lds_read_b128(q_ptr[ks] + so + kSlabBytes), lds_read_b128(k_ptr[ks] + kTileBytes), dp);
       }
       // does this wave's key block select the first / second 16 query rows of the slab?
       const bool on0 = !kTiled || ((bits_cmp >> (2 * kg)) & 1) != 0;
       const bool on1 = !kTiled || ((bits_cmp >> (2 * kg + 1)) & 1) != 0;
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const f32x4 l4 = *reinterpret_cast<const f32x4*>(smem + so + st_off + 32 * g);
+        const f32x4 l4 = lds_read_f32x4(st_ptr + so + 32 * g);
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           float pv = fast_exp2(__builtin_fmaf(s[4 * g + e], c, -l4[e]));
@@ -263,9 +264,9 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
 #pragma unroll
         for (int mb = 0; mb < 4; ++mb) {
           const int roff = so + 16 * j * kRowBytes;
-          const bf16x8 adv = cat(lds_read_tr(smem + kSlabBytes + roff, t_off[mb][0]), lds_read_tr(smem + kSlabBytes + roff, t_off[mb][1]));
+          const bf16x8 adv = cat(lds_read_tr(t_ptr[mb][0] + kSlabBytes + roff), lds_read_tr(t_ptr[mb][1] + kSlabBytes + roff));
           acc_v[mb] = mfma32(adv, pk[j], acc_v[mb]);
-          const bf16x8 adk = cat(lds_read_tr(smem + roff, t_off[mb][0]), lds_read_tr(smem + roff, t_off[mb][1]));
+          const bf16x8 adk = cat(lds_read_tr(t_ptr[mb][0] + roff), lds_read_tr(t_ptr[mb][1] + roff));
           acc_k[mb] = mfma32(adk, dsk[j], acc_k[mb]);
         }
     };

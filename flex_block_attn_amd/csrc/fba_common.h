@@ -55,6 +55,15 @@ FBA_DEVICE bf16x4 lds_read_tr(const char* base, int off) {
   return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((FBA_LDS bf16x4*)(base + off));
 }
 
+// The same fetches through pointers into LDS.  A per-lane address that is kept as such a pointer, with the base of the
+// work-group's LDS already folded in, goes into the fetch instruction as it is and constant displacements into its offset
+// field; an integer offset added to `smem` at every use costs a vector add per fetch instead.
+typedef const FBA_LDS char* LdsPtr;
+FBA_DEVICE LdsPtr lds_ptr(const void* p) { return (LdsPtr)p; }
+FBA_DEVICE bf16x8 lds_read_b128(LdsPtr p) { return *reinterpret_cast<const FBA_LDS bf16x8*>(p); }
+FBA_DEVICE f32x4 lds_read_f32x4(LdsPtr p) { return *reinterpret_cast<const FBA_LDS f32x4*>(p); }
+FBA_DEVICE bf16x4 lds_read_tr(LdsPtr p) { return __builtin_amdgcn_ds_read_tr16_b64_v4bf16((FBA_LDS bf16x4*)p); }
+
 FBA_DEVICE bf16x8 cat(bf16x4 lo, bf16x4 hi) { return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7); }
 
 // eight fp32 accumulators -> eight bf16 (round to nearest even)
