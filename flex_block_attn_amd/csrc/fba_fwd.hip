@@ -37,8 +37,7 @@ using IC = std::integral_constant<int, N>;
 struct FwdState {
   bf16x8 qreg[8];
   f32x16 acc_o[4];
-  f32x16 acc_l;  // every element of a lane: sum over keys of bf16(P) for the lane's query row
-  bf16x8 ones;
+  float l_run;  // sum over the keys this half-wave has seen of bf16(P) for the lane's query row
   float m_run;
   RowMajorOffsets rm;
   TransposedOffsets tr;
@@ -55,9 +54,7 @@ FBA_DEVICE f32x16 qk_half(const FwdState& st, const char* k_half) {
   return s;
 }
 
-// O^T += V^T P^T for 32 keys: 8 MFMAs, plus 2 with an all-ones A operand that accumulate the softmax denominator
-// (sum over keys of the same bf16 P that weighs V) without spending VALU additions on it.  Consecutive MFMAs go to
-// different accumulators.
+// O^T += V^T P^T for 32 keys: 8 MFMAs; consecutive MFMAs go to different accumulators.
 FBA_DEVICE void pv_half(FwdState& st, const char* v_half, const bf16x8 (&pk)[2]) {
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
@@ -67,7 +64,6 @@ FBA_DEVICE void pv_half(FwdState& st, const char* v_half, const bf16x8 (&pk)[2])
       const bf16x8 a = cat(lds_read_tr(v_half, st.tr.rd[mb][0] + roff), lds_read_tr(v_half, st.tr.rd[mb][1] + roff));
       st.acc_o[mb] = mfma32(a, pk[j], st.acc_o[mb]);
     }
-    st.acc_l = mfma32(st.ones, pk[j], st.acc_l);
   }
 }
 
@@ -84,8 +80,7 @@ FBA_DEVICE void softmax_reference(FwdState& st, const f32x16& s, bool active) {
     const float m_new = fmaxf(st.m_run, max_halves(mx));
     const float alpha = fast_exp2((st.m_run - m_new) * st.c);
     st.m_run = m_new;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) st.acc_l[r] *= alpha;
+    st.l_run *= alpha;
 #pragma unroll
     for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
@@ -105,6 +100,13 @@ FBA_DEVICE void softmax_exp(FwdState& st, f32x16& s, bf16x8 (&pk)[2], bool activ
 #pragma unroll
   for (int j = 0; j < 2; ++j)
     pk[j] = pack8(s[8 * j + 0], s[8 * j + 1], s[8 * j + 2], s[8 * j + 3], s[8 * j + 4], s[8 * j + 5], s[8 * j + 6], s[8 * j + 7]);
+  // denominator: the sum of the same bf16 P that weighs V, two values per dot-product instruction
+  const bf16x2 one2 = {(__bf16)1.f, (__bf16)1.f};
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      st.l_run = __builtin_amdgcn_fdot2_f32_bf16((bf16x2){pk[j][2 * t], pk[j][2 * t + 1]}, one2, st.l_run, false);
 }
 
 }  // namespace
@@ -148,10 +150,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   st.tr.init(lane);
   st.c = p.scale_log2e;
   st.m_run = kTiled ? -1e30f : -INFINITY;  // finite where whole slabs can be masked out, so that exp2 never sees inf - inf
-#pragma unroll
-  for (int t = 0; t < 8; ++t) st.ones[t] = (__bf16)1.f;
-#pragma unroll
-  for (int r = 0; r < 16; ++r) st.acc_l[r] = 0.f;
+  st.l_run = 0.f;
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb)
 #pragma unroll
@@ -275,7 +274,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 
   // epilogue: O = O^T / l, LSE = ln2 * (c m + log2 l)
   __bf16* orow = p.o + (qrow0 + l32) * kHeadDim;
-  const float l = st.acc_l[0];
+  const float l = sum_halves(st.l_run);
   const float inv = l > 0.f ? 1.f / l : 0.f;
   if (h == 0) p.lse[qrow0 + l32] = l > 0.f ? (st.m_run * st.c + __builtin_log2f(l)) * 0.6931471805599453f : -INFINITY;
 #pragma unroll
