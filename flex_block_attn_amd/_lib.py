@@ -30,6 +30,8 @@ SIGNATURES = {
     "fba_bwd_handover": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_ptr] * 9 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr]),
     "fba_bwd_dkdv_handover": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_ptr] * 3 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr]),
     "fba_bwd_dq_from_ds": (_c_i32, [_c_ptr] * 2 + [_c_i64] + [_c_ptr] * 5 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr]),
+    "fba_tile_slots": (_c_i32, [_c_ptr, _c_ptr, _c_i64, _c_i32, _c_i32, _c_ptr, _c_ptr, _c_ptr, _c_ptr]),
+    "fba_bwd_tiled_handover": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_ptr] * 10 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr]),
     "fba_bwd_noalloc": (_c_i32, [_c_ptr] * 13 + [_c_i64] + [_c_i32] * 8 + [_c_ptr]),
     "fba_tile_lists": (_c_i32, [_c_ptr, _c_i64, _c_i32, _c_i32, _c_i32, _c_i32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr]),
     "fba_block_mean": (_c_i32, [_c_ptr, _c_ptr, _c_i64, _c_i32, _c_i32, _c_i32, _c_ptr]),

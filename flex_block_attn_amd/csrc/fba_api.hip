@@ -358,6 +358,49 @@ int32_t fba_bwd_handover(const void* q, const void* k, const void* v, const void
                             q_block, k_block, hip_stream);
 }
 
+int32_t fba_tile_slots(const int32_t* kt_cnt, const int32_t* kt_ent, int64_t mask_bh, int32_t n_qt, int32_t n_kt, int32_t* pair_base,
+                       int32_t* kt_slot, int32_t* slot_table, void* hip_stream) {
+  if (mask_bh <= 0 || n_qt <= 0 || n_kt <= 0)
+    return fail(FBA_ERR_INVALID, "mask_bh, n_qt, n_kt must be positive (got %lld %d %d)", (long long)mask_bh, n_qt, n_kt);
+  if (mask_bh * (int64_t)n_kt * n_qt * 4 > 0x7fffffffLL) return fail(FBA_ERR_INVALID, "more than 2^31 tile-list entries");
+  if (!kt_cnt || !kt_ent || !pair_base || !kt_slot || !slot_table) return fail(FBA_ERR_INVALID, "null pointer argument");
+  hipError_t e = fba::launch_tile_slots(kt_cnt, kt_ent, mask_bh, n_qt, n_kt, 4 * n_qt, pair_base, kt_slot, slot_table, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "tile_slots launch");
+}
+
+int32_t fba_bwd_tiled_handover(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse, float* stats,
+                               void* ds_ws, int64_t ds_ws_bytes, void* dq, void* dk, void* dv, const int32_t* qt_cnt,
+                               const int32_t* qt_ent, const int32_t* kt_cnt, const int32_t* kt_ent, const int32_t* pair_base,
+                               const int32_t* kt_slot, const int32_t* slot_table, int64_t n_pairs, int64_t mask_bh, int32_t B,
+                               int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,
+                               void* hip_stream) {
+  const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
+  if (int rc = check_shape(s)) return rc;
+  if (int rc = check_lists(s, true, "backward")) return rc;
+  // everything is validated before the first launch, so that a rejected call leaves nothing on the stream
+  if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"o", o}, {"d_o", d_o}, {"dq", dq}, {"dk", dk}, {"dv", dv}, {"ds_ws", ds_ws}})) return rc;
+  if (!lse || !stats || !qt_cnt || !qt_ent || !kt_cnt || !kt_ent || !pair_base || !kt_slot || !slot_table)
+    return fail(FBA_ERR_INVALID, "null pointer argument");
+  if ((int64_t)B * Hq * Sq >= (1LL << 30)) return fail(FBA_ERR_INVALID, "B*Hq*Sq must be below 2^30");
+  if (n_pairs < 0) return fail(FBA_ERR_INVALID, "n_pairs must not be negative");
+  const int64_t need = n_pairs * 128 * 128 * 2;
+  if (ds_ws_bytes < need)
+    return fail(FBA_ERR_INVALID, "backward: ds_ws holds %lld bytes, %lld tile pairs of 128 x 128 need %lld", (long long)ds_ws_bytes,
+                (long long)n_pairs, (long long)need);
+  if (int rc = fba_bwd_stats(o, d_o, lse, stats, (int64_t)B * Hq * Sq, head_dim, hip_stream)) return rc;
+  fba::BwdParams p{};
+  fill_bwd(p, s);
+  p.tiled = 1;
+  p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.d_o = (const __bf16*)d_o;
+  p.stats = stats; p.dq = (__bf16*)dq; p.dk = (__bf16*)dk; p.dv = (__bf16*)dv;
+  p.q_cnt = qt_cnt; p.q_idx = qt_ent; p.k_cnt = kt_cnt; p.k_idx = kt_ent;
+  p.ds_ws = (__bf16*)ds_ws; p.pair_base = pair_base; p.k_slot = kt_slot; p.q_slot = slot_table;
+  hipError_t e = fba::launch_bwd_dkdv(p, (hipStream_t)hip_stream);
+  if (e != hipSuccess) return hip_fail(e, "dkdv (tile lists, hand-over) launch");
+  e = fba::launch_bwd_dq_from_ds(p, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "dq (from dS, tile lists) launch");
+}
+
 }  // extern "C"
 
 namespace {

@@ -43,11 +43,11 @@ using IC = std::integral_constant<int, N>;
 
 // kTiled = false: q_block and k_block are multiples of 128; list entries are query blocks, expanded to q_block/32 slabs.
 // kTiled = true: tile lists; list entries are 32-row query slabs with a predicate per (key group, 16-row half-slab).
-// kHandOver (block lists only): every wave also stores the bf16 dS it forms to p.ds_ws (layout: fba_common.h), so that
-// dQ = dS K can be formed later without recomputing S and dP.
+// kHandOver: every wave also stores the bf16 dS it forms to p.ds_ws (layout: fba_common.h), so that dQ = dS K can be
+// formed later without recomputing S and dP.  With tile lists the workspace is divided into (128-row query tile, 128-key
+// tile) pairs and a wave that leaves a slab out stores nothing for it.
 template <bool kTiled, bool kHandOver>
 __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_per_eu(2, 2))) void dkdv_kernel(const BwdParams p) {
-  static_assert(!(kTiled && kHandOver), "dS hand-over works on block lists");
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int TK = 128;
 
@@ -147,8 +147,10 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     request_pair(1);
 
     // tile lists: predicate bits of this wave's slab, from a second walk over the same lists (two entries per step)
-    int g_cmp = -1, e_cmp = -1, cnt_cmp = 0, bits_cmp = 0;
-    ConstIdx idx_cmp = nullptr;
+    // (with the hand-over also the entry's tile-pair number and its slab inside the query tile)
+    int g_cmp = -1, e_cmp = -1, cnt_cmp = 0, bits_cmp = 0, sub_cmp = 0;
+    int64_t slot_cmp = 0, head_slot0 = 0;
+    ConstIdx idx_cmp = nullptr, slot_idx_cmp = nullptr;
     auto next_bits = [&]() {
       ++e_cmp;
       while (e_cmp >= cnt_cmp) {
@@ -156,9 +158,19 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
         const int64_t lr = list_row(g_cmp);
         cnt_cmp = k_cnt[lr];
         idx_cmp = const_idx(p.k_idx + lr * row_len);
+        if constexpr (kHandOver) {
+          slot_idx_cmp = const_idx(p.k_slot + lr * row_len);
+          const int64_t bh = (int64_t)b * p.Hq + hkv * group + g_cmp;
+          head_slot0 = p.mask_bh == 1 ? bh * const_idx(p.pair_base)[tiles_per_head] : 0;
+        }
         e_cmp = 0;
       }
-      bits_cmp = idx_cmp[e_cmp] & 255;
+      const int ent = idx_cmp[e_cmp];
+      bits_cmp = ent & 255;
+      if constexpr (kHandOver) {
+        sub_cmp = (ent >> 8) & 3;
+        slot_cmp = head_slot0 + slot_idx_cmp[e_cmp];
+      }
     };
     if constexpr (kTiled) {
       next_bits();
@@ -191,7 +203,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
         ho_next_entry();
       }
     };
-    if constexpr (kHandOver) {
+    if constexpr (kHandOver && !kTiled) {
       ho_next_entry();
       ho_advance(par);
     }
@@ -252,8 +264,11 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
         dsk[j] = pack8(dp[8 * j + 0], dp[8 * j + 1], dp[8 * j + 2], dp[8 * j + 3], dp[8 * j + 4], dp[8 * j + 5], dp[8 * j + 6], dp[8 * j + 7]);
       }
       if constexpr (kHandOver) {
-        char* unit = reinterpret_cast<char*>(p.ds_ws) + (h_slot0 + h_e) * pair_bytes +
-                     ((int64_t)((h_s >> 2) * nsub_k + t_key) * 4 + (h_s & 3)) * kDsUnitBytes;
+        char* unit = reinterpret_cast<char*>(p.ds_ws);
+        if constexpr (kTiled)  // 16 units per tile pair, ordered (32-key slab, 32-row slab)
+          unit += slot_cmp * (16 * kDsUnitBytes) + (kg * 4 + sub_cmp) * kDsUnitBytes;
+        else
+          unit += (h_slot0 + h_e) * pair_bytes + ((int64_t)((h_s >> 2) * nsub_k + t_key) * 4 + (h_s & 3)) * kDsUnitBytes;
         // written once, read once by another kernel much later: streaming stores, so that they do not push the Q / dO
         // slabs that other work-groups are about to fetch out of L2
         __builtin_nontemporal_store(dsk[0], reinterpret_cast<bf16x8*>(unit + ho_off0));
@@ -274,12 +289,14 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     const int npairs = (nslabs + 1) >> 1;
     auto step = [&](auto half_c, int s2) {
       // tile lists: a wave whose 32 keys are selected by neither half of the slab leaves the slab out (wave-uniform)
-      if (2 * s2 + par < nslabs && (!kTiled || ((bits_cmp >> (2 * kg)) & 3) != 0)) compute(half_c);
+      const bool worked = 2 * s2 + par < nslabs && (!kTiled || ((bits_cmp >> (2 * kg)) & 3) != 0);
+      if (worked) compute(half_c);
       if constexpr (kTiled) { next_bits(); next_bits(); }
-      if constexpr (kHandOver) ho_advance(2);
-      // this wave's copies of the next pair, requested one step ago, must have landed.  The two dS stores of this step are
-      // younger and may still be on their way (the counter covers loads and stores alike and runs down in issue order).
-      if constexpr (kHandOver) wait_vmem<2>(); else wait_vmem<0>();
+      if constexpr (kHandOver && !kTiled) ho_advance(2);
+      // this wave's copies of the next pair, requested one step ago, must have landed.  The two dS stores of this step, if
+      // the wave made any, are younger and may still be on their way (the counter covers loads and stores alike and runs
+      // down in issue order).
+      if (kHandOver && worked) wait_vmem<2>(); else wait_vmem<0>();
       __syncthreads();  // everybody is done with this pair and everybody's copies of the next pair have landed
       request_pair(decltype(half_c)::value);
     };
@@ -330,8 +347,8 @@ hipError_t launch_bwd_dkdv(BwdParams p, hipStream_t stream) {
   p.num_items = p.B * p.Hkv * (p.Skv / 128);
   p.items_per_xcd = (p.num_items + kNumXcd - 1) / kNumXcd;
   const bool hand_over = p.ds_ws != nullptr;
-  if (hand_over && p.tiled) return hipErrorInvalidValue;
-  void (*fn)(const BwdParams) = p.tiled ? &dkdv_kernel<true, false> : hand_over ? &dkdv_kernel<false, true> : &dkdv_kernel<false, false>;
+  void (*fn)(const BwdParams) = p.tiled ? (hand_over ? &dkdv_kernel<true, true> : &dkdv_kernel<true, false>)
+                                        : (hand_over ? &dkdv_kernel<false, true> : &dkdv_kernel<false, false>);
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(fn, dim3(p.items_per_xcd * kNumXcd), dim3(512), kSmemBytes, stream, p);

@@ -12,6 +12,12 @@
 // The kernel does 8 MFMAs per 16 KiB it reads, so it runs at the speed of memory: K slabs (8 KiB, shared by the four
 // waves, mostly L2 hits) and dS units (2 KiB per wave, each read exactly once from HBM) travel global -> LDS directly
 // into a ring of four stages; stage t+4 is requested when stage t is dead.
+//
+// kTiled: tile lists.  The workspace is divided into (128-row query tile, 128-key tile) pairs of 16 units; the list of the
+// work-group's query tile names key blocks with a predicate per 16 rows.  A wave whose rows do not select a key block has
+// no unit there (the key-major kernel stored none): it copies 2 KiB of zeros instead, so that every wave issues the same
+// number of copies per stage, and leaves the matrix work of those steps out.
+#include <mutex>
 #include <type_traits>
 
 #include "fba_common.h"
@@ -31,6 +37,7 @@ using IC = std::integral_constant<int, N>;
 
 }  // namespace
 
+template <bool kTiled>
 __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_per_eu(2, 2))) void dq_from_ds_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];  // ring [4] of (K slab | dS units)
   constexpr int TQ = 128;
@@ -49,17 +56,22 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   const char* kp = reinterpret_cast<const char*>(p.k + ((int64_t)(b * p.Hkv + hkv) * p.Skv) * kHeadDim);
 
   const int qblk = (qt * TQ) / p.q_block;
-  const int tq = (qt * TQ - qblk * p.q_block) / TQ;  // this tile's position inside its query block
-  const int64_t mrow = (p.mask_bh == 1 ? 0 : (int64_t)bh) * p.nQ + qblk;
+  const int tq = kTiled ? 0 : (qt * TQ - qblk * p.q_block) / TQ;  // this tile's position inside its query block
+  const int n_kt = p.Skv / 128;
+  const int64_t mrow = (p.mask_bh == 1 ? 0 : (int64_t)bh) * (kTiled ? tiles_per_head : p.nQ) + (kTiled ? qt : qblk);
   const int cnt = p.q_cnt[mrow];
   const ConstIdx idx = const_idx(p.q_idx + mrow * p.nK);
-  const ConstIdx slot = const_idx(p.q_slot + mrow * p.nK);
+  // block lists: pair number per list entry; tile lists: pair number per key tile, for this query tile
+  const ConstIdx slot = const_idx(p.q_slot + mrow * (kTiled ? n_kt : p.nK));
   const int nsub = p.k_block / kSlab;
   const int nsteps = cnt * nsub;
-  const int64_t pair_bytes = (int64_t)p.q_block * p.k_block * 2;
-  // dS of this wave's 32 rows: pair base + (tq * nsub + t) * 4 units + wave, t = 32-key slab inside the key block
-  const int64_t head_pairs = p.mask_bh == 1 ? (int64_t)bh * const_idx(p.pair_base)[p.nK] : 0;
+  const int64_t pair_bytes = kTiled ? 16 * kDsUnitBytes : (int64_t)p.q_block * p.k_block * 2;
+  // dS of this wave's 32 rows: pair base + (tq * nsub + t) * 4 units + wave, t = 32-key slab inside the key block (inside
+  // the key tile with tile lists)
+  const int64_t head_pairs = p.mask_bh == 1 ? (int64_t)bh * const_idx(p.pair_base)[kTiled ? n_kt : p.nK] : 0;
   const char* ds_base = reinterpret_cast<const char*>(p.ds_ws) + head_pairs * pair_bytes + ((int64_t)tq * nsub * 4 + wave) * kDsUnitBytes;
+  auto key_block = [&](int e) -> int { return kTiled ? idx[e] >> 8 : idx[e]; };
+  const int wave_bits = 3 << (2 * wave);  // predicate bits of this wave's two 16-row groups in a tile-list entry
 
   TransposedOffsets tr;
   tr.init(lane);
@@ -87,27 +99,40 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   // sources of the next stage to request, in list order; the following list entry is read one block ahead
   const int64_t block_bytes = (int64_t)p.k_block * kRowBytes;
   int e_next = 1, rem = nsub;
-  int64_t k_off = cnt > 0 ? idx[0] * block_bytes : 0;
-  int64_t ds_off_g = cnt > 0 ? slot[0] * pair_bytes : 0;
-  int blk_next = cnt > 1 ? idx[1] : 0;
-  int slot_next = cnt > 1 ? slot[1] : 0;
+  int64_t k_off = cnt > 0 ? key_block(0) * block_bytes : 0;
+  int64_t ds_off_g = cnt > 0 && !kTiled ? slot[0] * pair_bytes : 0;
+  int blk_next = cnt > 1 ? key_block(1) : 0;
+  int slot_next = cnt > 1 && !kTiled ? slot[1] : 0;
+  // tile lists: predicate bits of the entry being requested and of the next one; pair number of the key tile that the
+  // next stage's slab lies in, read one stage ahead
+  int bits_req = kTiled && cnt > 0 ? idx[0] & 255 : 0;
+  int bits_req_next = kTiled && cnt > 1 ? idx[1] & 255 : 0;
+  int tile_slot = kTiled && cnt > 0 ? slot[(int)(k_off >> 15)] : 0;  // 32 KiB of K rows per key tile
   const uint32_t lane16 = (uint32_t)lane * 16;
   auto copy_next = [&](int ring) {
     const uint32_t dst = ring_dst + ring * kStageBytes;
     dma.copy(dst, kp + k_off);
-    dma16_stream(dst + kSlabBytes + wave * kDsUnitBytes, ds_base + ds_off_g, lane16);
-    dma16_stream(dst + kSlabBytes + wave * kDsUnitBytes + 1024, ds_base + ds_off_g, lane16 + 1024);
+    const char* src = ds_base + ds_off_g;
+    if constexpr (kTiled) {
+      const int t = (int)(k_off >> 13) & 3;  // 32-key slab inside its key tile
+      src = (bits_req & wave_bits) != 0 ? ds_base + (int64_t)tile_slot * pair_bytes + t * (4 * kDsUnitBytes) : p.zero_unit;
+    }
+    dma16_stream(dst + kSlabBytes + wave * kDsUnitBytes, src, lane16);
+    dma16_stream(dst + kSlabBytes + wave * kDsUnitBytes + 1024, src, lane16 + 1024);
     if (--rem == 0) {
       rem = nsub;
       k_off = blk_next * block_bytes;
       ds_off_g = slot_next * pair_bytes;
+      bits_req = bits_req_next;
       ++e_next;
-      blk_next = e_next < cnt ? idx[e_next] : 0;
-      slot_next = e_next < cnt ? slot[e_next] : 0;
+      blk_next = e_next < cnt ? key_block(e_next) : 0;
+      if constexpr (kTiled) bits_req_next = e_next < cnt ? idx[e_next] & 255 : 0;
+      else slot_next = e_next < cnt ? slot[e_next] : 0;
     } else {
       k_off += kSlabBytes;
       ds_off_g += 4 * kDsUnitBytes;
     }
+    if constexpr (kTiled) tile_slot = slot[(int)(k_off >> 15)];  // past the last stage: some listed tile's number, unused
   };
 
   if (nsteps > 0) {
@@ -117,18 +142,33 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     wait_vmem<0>();
     __syncthreads();
 
+    // tile lists: predicate bits of the entry whose slab is worked on (a second walk over the list)
+    int e_cmp = 0, rem_cmp = nsub;
+    int bits_cmp = kTiled ? idx[0] & 255 : 255;
+    int bits_ahead = kTiled && cnt > 1 ? idx[1] & 255 : 0;
+
     // step t (t % 4 == R): dQ += K_t^T dS_t
     auto step = [&](auto ring_c, int t) {
       constexpr int R = decltype(ring_c)::value;
       const char* stage = smem + R * kStageBytes;
+      if (!kTiled || (bits_cmp & wave_bits) != 0) {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const bf16x8 dsk = cat(lds_read_tr(stage, ds_off[j][0]), lds_read_tr(stage, ds_off[j][1]));
+        for (int j = 0; j < 2; ++j) {
+          const bf16x8 dsk = cat(lds_read_tr(stage, ds_off[j][0]), lds_read_tr(stage, ds_off[j][1]));
 #pragma unroll
-        for (int mb = 0; mb < 4; ++mb) {
-          const int roff = 16 * j * kRowBytes;
-          const bf16x8 a = cat(lds_read_tr(stage, tr.rd[mb][0] + roff), lds_read_tr(stage, tr.rd[mb][1] + roff));
-          acc[mb] = mfma32(a, dsk, acc[mb]);
+          for (int mb = 0; mb < 4; ++mb) {
+            const int roff = 16 * j * kRowBytes;
+            const bf16x8 a = cat(lds_read_tr(stage, tr.rd[mb][0] + roff), lds_read_tr(stage, tr.rd[mb][1] + roff));
+            acc[mb] = mfma32(a, dsk, acc[mb]);
+          }
+        }
+      }
+      if constexpr (kTiled) {
+        if (--rem_cmp == 0) {
+          rem_cmp = nsub;
+          ++e_cmp;
+          bits_cmp = bits_ahead;
+          bits_ahead = e_cmp + 1 < cnt ? idx[e_cmp + 1] & 255 : 0;
         }
       }
       // stage t+1 must have landed (first read in step t+1); the copies of stages t+2 and t+3 (4 each) may still fly
@@ -155,14 +195,44 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     }
 }
 
+namespace {
+
+// What a wave copies in place of a dS unit that nobody stored (tile lists).  Part of the library's device image and never
+// written; host code reaches it only through the address hipGetSymbolAddress returns for the current device.
+__device__ __attribute__((aligned(256))) char g_zero_unit[kDsUnitBytes];
+
+hipError_t zero_unit_address(const char** out) {
+  constexpr int kMaxDevices = 64;
+  static std::mutex mu;
+  static const char* cache[kMaxDevices] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  if (dev < 0 || dev >= kMaxDevices) return hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> lock(mu);
+  if (cache[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_zero_unit));
+    if (e != hipSuccess) return e;
+    cache[dev] = static_cast<const char*>(ptr);
+  }
+  *out = cache[dev];
+  return hipSuccess;
+}
+
+}  // namespace
+
 hipError_t launch_bwd_dq_from_ds(BwdParams p, hipStream_t stream) {
   constexpr int kSmem = kRing * kStageBytes;
-  if (p.tiled || p.ds_ws == nullptr) return hipErrorInvalidValue;
+  if (p.ds_ws == nullptr) return hipErrorInvalidValue;
   p.num_items = p.B * p.Hq * (p.Sq / 128);
   p.items_per_xcd = (p.num_items + kNumXcd - 1) / kNumXcd;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&dq_from_ds_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
+  void (*fn)(const BwdParams) = p.tiled ? &dq_from_ds_kernel<true> : &dq_from_ds_kernel<false>;
+  hipError_t e = hipSuccess;
+  if (p.tiled && (e = zero_unit_address(&p.zero_unit)) != hipSuccess) return e;
+  e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(dq_from_ds_kernel, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
+  hipLaunchKernelGGL(fn, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
   return hipGetLastError();
 }
 

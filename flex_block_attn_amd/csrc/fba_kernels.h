@@ -49,15 +49,22 @@ struct BwdParams {
   // tiled = 1: q_cnt / q_idx are qt_cnt / qt_ent and k_cnt / k_idx are kt_cnt [mask_bh, Skv/128] /
   // kt_ent [mask_bh, Skv/128, Sq/32] (see tile_lists_kernel)
   int tiled;
-  // dS hand-over (block lists only; null when unused).  The key-major kernel stores dS of every selected block pair
-  // into ds_ws and the query-major kernel reads it back instead of recomputing S and dP.
+  // dS hand-over (null when unused).  The key-major kernel stores dS of every selected block pair into ds_ws and the
+  // query-major kernel reads it back instead of recomputing S and dP.  Block lists:
   //   pair_base [mask_bh * nK + 1]: exclusive prefix sum of k_cnt; the last entry is the number of pairs in the lists
   //   q_slot    [mask_bh, nQ, nK]:  pair number of entry e of query block I, i.e. pair_base[m, J] + position of I in
   //                                 k_idx[m, J, :] for J = q_idx[m, I, e]; -1 beyond q_cnt
   // Pair n of head bh lives at ds_ws + (n + (mask_bh == 1 ? bh * pairs : 0)) * q_block * k_block * 2 bytes.
+  // Tile lists (see tile_slots_kernel): the pairs are (128-row query tile, 128-key tile) pairs of 32 KiB,
+  //   pair_base [mask_bh * Skv/128 + 1]:        exclusive prefix sum of the listed tile pairs per key tile
+  //   k_slot    [mask_bh, Skv/128, Sq/32]:      pair number of every kt_ent entry
+  //   q_slot    [mask_bh, Sq/128, Skv/128]:     pair number of (query tile, key tile), -1 where nothing is listed
+  //   zero_unit: 2 KiB of zeros in device memory, read in place of a dS unit that no wave stored
   __bf16* ds_ws;
   const int32_t* pair_base;
   const int32_t* q_slot;
+  const int32_t* k_slot;
+  const char* zero_unit;
 };
 
 hipError_t launch_mask_compact(const uint8_t* mask, int64_t mask_bh, int nQ, int nK, int32_t* q_cnt, int32_t* q_idx,
@@ -78,5 +85,7 @@ hipError_t launch_bwd_dq_from_ds(BwdParams p, hipStream_t stream);
 hipError_t launch_probe_mfma(const float* src, float* sink, int work_groups, int iters, hipStream_t stream);
 hipError_t launch_pair_slots(const int32_t* q_cnt, const int32_t* q_idx, const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh,
                              int nQ, int nK, int32_t* pair_base, int32_t* q_slot, hipStream_t stream);
+hipError_t launch_tile_slots(const int32_t* kt_cnt, const int32_t* kt_ent, int64_t mask_bh, int n_qt, int n_kt, int n_qs,
+                             int32_t* pair_base, int32_t* kt_slot, int32_t* slot_table, hipStream_t stream);
 
 }  // namespace fba

@@ -185,6 +185,74 @@ hipError_t launch_pair_slots(const int32_t* q_cnt, const int32_t* q_idx, const i
   return hipGetLastError();
 }
 
+// Tile-pair numbering for the dS hand-over on tile lists.  The unit of the workspace is a (128-row query tile T, 128-key
+// tile U) pair, listed when some 32-row slab of T appears in kt_ent[m, U, :]; pairs are numbered in key-major order:
+// pair_base = exclusive prefix sum of the listed pairs per (m, U) row (last entry = total), pair (m, U, r) =
+// pair_base[m, U] + r for the r-th distinct query tile of the ascending row.  kt_slot gives every kt_ent entry the number
+// of its pair (what the key-major kernel needs, next to the entry); slot_table [m, T, U] gives the query-major kernel
+// the same number by position (-1 where nothing is listed).  One wave per row; integer work, independent of scheduling.
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void tile_pair_count_kernel(
+    const int32_t* __restrict__ kt_cnt, const int32_t* __restrict__ kt_ent, int64_t rows, int n_qs, int32_t* __restrict__ row_cnt) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int cnt = kt_cnt[row];
+  const int32_t* list = kt_ent + row * n_qs;
+  int total = 0;
+  for (int t0 = 0; t0 < cnt; t0 += 64) {
+    const int e = t0 + lane;
+    const bool first = e < cnt && (e == 0 || (list[e] >> 10) != (list[e - 1] >> 10));  // entry = slab << 8 | bits, tile = slab / 4
+    total += __popcll(__ballot(first));
+  }
+  if (lane == 0) row_cnt[row] = total;
+}
+
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void fill_i32_kernel(int32_t* __restrict__ out, int64_t n, int32_t value) {
+  for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < n; t += (int64_t)gridDim.x * 256) out[t] = value;
+}
+
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void tile_slots_kernel(
+    const int32_t* __restrict__ kt_cnt, const int32_t* __restrict__ kt_ent, const int32_t* __restrict__ pair_base, int64_t rows,
+    int n_qt, int n_kt, int n_qs, int32_t* __restrict__ kt_slot, int32_t* __restrict__ slot_table) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int64_t m = row / n_kt;
+  const int U = (int)(row - m * n_kt);
+  const int cnt = kt_cnt[row];
+  const int32_t* list = kt_ent + row * n_qs;
+  const int32_t base = pair_base[row];
+  int seen = 0;  // distinct query tiles before this chunk
+  for (int t0 = 0; t0 < n_qs; t0 += 64) {
+    const int e = t0 + lane;
+    const bool in = e < cnt;
+    const int T = in ? list[e] >> 10 : 0;
+    const bool first = in && (e == 0 || (list[e - 1] >> 10) != T);
+    const unsigned long long bal = __ballot(first);
+    const int32_t slot = base + seen + __popcll(bal & (~0ull >> (63 - lane))) - 1;  // firsts up to and including this lane
+    if (e < n_qs) kt_slot[row * n_qs + e] = in ? slot : -1;
+    if (first) slot_table[(m * n_qt + T) * n_kt + U] = slot;
+    seen += __popcll(bal);
+  }
+}
+
+hipError_t launch_tile_slots(const int32_t* kt_cnt, const int32_t* kt_ent, int64_t mask_bh, int n_qt, int n_kt, int n_qs,
+                             int32_t* pair_base, int32_t* kt_slot, int32_t* slot_table, hipStream_t stream) {
+  const int64_t rows = mask_bh * n_kt, table = mask_bh * n_qt * n_kt;
+  if (rows <= 0 || table <= 0 || n_qs <= 0) return hipSuccess;
+  const int64_t blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffffLL) return hipErrorInvalidValue;
+  // the per-row counts rest in the first `rows` entries of kt_slot (which has rows * n_qs >= rows entries) until the
+  // prefix sum has read them
+  hipLaunchKernelGGL(tile_pair_count_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, kt_cnt, kt_ent, rows, n_qs, kt_slot);
+  hipLaunchKernelGGL(pair_base_kernel, dim3(1), dim3(1024), 0, stream, kt_slot, rows, pair_base);
+  const int64_t fill_blocks = (table + 255) / 256;
+  hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)(fill_blocks < 4096 ? fill_blocks : 4096)), dim3(256), 0, stream, slot_table, table, -1);
+  hipLaunchKernelGGL(tile_slots_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, kt_cnt, kt_ent, pair_base, rows, n_qt, n_kt, n_qs,
+                     kt_slot, slot_table);
+  return hipGetLastError();
+}
+
 // Backward statistics, one pass over O and dO: stats[r] = lse[r] * log2(e) and stats[rows + r] = -delta[r] =
 // -sum_c dO[r, c] * O[r, c] in fp32 (reference: bwd_attend_prep_ker, flex_block_attn_h100.cu:375-379).  The backward
 // kernels exponentiate in base 2, hence the pre-scaled LSE; they start the dP accumulators from the second plane, so that

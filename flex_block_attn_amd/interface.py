@@ -42,9 +42,12 @@ class BlockLists:
     nQ: int
     nK: int
     tiled: bool = False
-    # pair numbering for the dS hand-over of backward (fba_pair_slots), filled by `number_pairs`
-    pair_base: Optional[torch.Tensor] = None  # [mask_bh * nK + 1] int32; the last entry is the number of listed pairs
-    q_slot: Optional[torch.Tensor] = None     # [mask_bh, nQ, nK] int32
+    # pair numbering for the dS hand-over of backward, filled by `number_pairs`.  Block lists (fba_pair_slots):
+    # pair_base [mask_bh * nK + 1], q_slot [mask_bh, nQ, nK].  Tile lists (fba_tile_slots): pair_base
+    # [mask_bh * Skv/128 + 1], q_slot [mask_bh, Sq/128, Skv/128] (the slot table), k_slot [mask_bh, Skv/128, Sq/32].
+    pair_base: Optional[torch.Tensor] = None  # int32; the last entry is the number of listed pairs
+    q_slot: Optional[torch.Tensor] = None     # int32
+    k_slot: Optional[torch.Tensor] = None     # int32, tile lists only
     _count: Optional[tuple] = None            # (pinned host copy of pair_base[-1], event recorded after the copy)
 
     def listed_pairs(self):
@@ -103,8 +106,9 @@ def needs_tile_lists(q_block_size, kv_block_size):
     return q_block_size % 128 != 0 or kv_block_size % 128 != 0
 
 
-def tile_block_mask(block_mask, q_block_size, kv_block_size):
-    """bool block mask -> tile lists (a BlockLists with `tiled` set), via fba_tile_lists."""
+def tile_block_mask(block_mask, q_block_size, kv_block_size, with_pair_numbers=False):
+    """bool block mask -> tile lists (a BlockLists with `tiled` set), via fba_tile_lists.  `with_pair_numbers` also
+    numbers the tile pairs right away (see `number_pairs`)."""
     if block_mask.dtype != torch.bool:
         raise TypeError(f"block_mask must be a bool tensor, got {block_mask.dtype}")
     if block_mask.dim() not in (2, 4):
@@ -124,13 +128,14 @@ def tile_block_mask(block_mask, q_block_size, kv_block_size):
     with torch.cuda.device(m.device):
         _lib.call("fba_tile_lists", _ptr(m), mask_bh, nQ, nK, q_block_size, kv_block_size, _ptr(qt_cnt), _ptr(qt_ent),
                   _ptr(kt_cnt), _ptr(kt_ent), _stream())
-    return BlockLists(qt_cnt, qt_ent, kt_cnt, kt_ent, mask_bh, nQ, nK, tiled=True)
+    lists = BlockLists(qt_cnt, qt_ent, kt_cnt, kt_ent, mask_bh, nQ, nK, tiled=True)
+    return number_pairs(lists) if with_pair_numbers else lists
 
 
 def lists_for(block_mask, q_block_size, kv_block_size, with_pair_numbers=False):
     """The list flavour the kernels need for these block sizes."""
     if needs_tile_lists(q_block_size, kv_block_size):
-        return tile_block_mask(block_mask, q_block_size, kv_block_size)
+        return tile_block_mask(block_mask, q_block_size, kv_block_size, with_pair_numbers)
     return compact_block_mask(block_mask, with_pair_numbers)
 
 
@@ -197,7 +202,11 @@ def _check_lists(lists, q, B, Hq, Sq, Skv, q_block_size, kv_block_size):
     else:
         shapes = ((M, lists.nQ), (M, lists.nQ, lists.nK), (M, lists.nK), (M, lists.nK, lists.nQ))
     names, tensors = ["q_cnt", "q_idx", "k_cnt", "k_idx"], [lists.q_cnt, lists.q_idx, lists.k_cnt, lists.k_idx]
-    if lists.pair_base is not None:
+    if lists.pair_base is not None and lists.tiled:
+        names += ["pair_base", "q_slot", "k_slot"]
+        tensors += [lists.pair_base, lists.q_slot, lists.k_slot]
+        shapes += ((M * (Skv // 128) + 1,), (M, Sq // 128, Skv // 128), (M, Skv // 128, Sq // 32))
+    elif lists.pair_base is not None:
         names += ["pair_base", "q_slot"]
         tensors += [lists.pair_base, lists.q_slot]
         shapes += ((M * lists.nK + 1,), (M, lists.nQ, lists.nK))
@@ -222,23 +231,31 @@ def forward_with_lists(q, k, v, q_block_size, kv_block_size, lists):
 
 
 def number_pairs(lists):
-    """Pair numbering of block lists for the dS hand-over (fba_pair_slots), kept on `lists`.  The number of listed
-    pairs, which sizes the workspace, is copied to pinned host memory asynchronously; `lists.listed_pairs()` waits for
-    that copy alone."""
-    if lists.tiled:
-        raise ValueError("the dS hand-over works on block lists, not tile lists")
+    """Pair numbering for the dS hand-over, kept on `lists`: block pairs of block lists (fba_pair_slots), pairs of
+    128-row tiles of tile lists (fba_tile_slots).  The number of listed pairs, which sizes the workspace, is copied to
+    pinned host memory asynchronously; `lists.listed_pairs()` waits for that copy alone."""
     if lists.pair_base is None:
         dev = lists.k_cnt.device
-        pair_base = torch.empty((lists.mask_bh * lists.nK + 1,), dtype=torch.int32, device=dev)
-        q_slot = torch.empty((lists.mask_bh, lists.nQ, lists.nK), dtype=torch.int32, device=dev)
+        i32 = dict(dtype=torch.int32, device=dev)
         host = torch.empty((1,), dtype=torch.int32, pin_memory=True)
+        k_slot = None
         with torch.cuda.device(dev):
-            _lib.call("fba_pair_slots", _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), lists.mask_bh,
-                      lists.nQ, lists.nK, _ptr(pair_base), _ptr(q_slot), _stream())
+            if lists.tiled:
+                n_qt, n_kt = lists.q_cnt.shape[1], lists.k_cnt.shape[1]
+                pair_base = torch.empty((lists.mask_bh * n_kt + 1,), **i32)
+                q_slot = torch.empty((lists.mask_bh, n_qt, n_kt), **i32)
+                k_slot = torch.empty((lists.mask_bh, n_kt, 4 * n_qt), **i32)
+                _lib.call("fba_tile_slots", _ptr(lists.k_cnt), _ptr(lists.k_idx), lists.mask_bh, n_qt, n_kt, _ptr(pair_base),
+                          _ptr(k_slot), _ptr(q_slot), _stream())
+            else:
+                pair_base = torch.empty((lists.mask_bh * lists.nK + 1,), **i32)
+                q_slot = torch.empty((lists.mask_bh, lists.nQ, lists.nK), **i32)
+                _lib.call("fba_pair_slots", _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), lists.mask_bh,
+                          lists.nQ, lists.nK, _ptr(pair_base), _ptr(q_slot), _stream())
             host.copy_(pair_base[-1:], non_blocking=True)
             event = torch.cuda.Event()
             event.record()
-        lists.pair_base, lists.q_slot, lists._count = pair_base, q_slot, (host, event)
+        lists.pair_base, lists.q_slot, lists.k_slot, lists._count = pair_base, q_slot, k_slot, (host, event)
     return lists
 
 
@@ -251,15 +268,16 @@ def ds_workspace_bytes(lists, B, Hq, q_block_size, kv_block_size):
     """(pairs over all heads, bytes of dS workspace) the hand-over backward needs for these lists."""
     listed = number_pairs(lists).listed_pairs()
     pairs = listed * (B * Hq if lists.mask_bh == 1 else 1)
-    return pairs, pairs * q_block_size * kv_block_size * 2
+    return pairs, pairs * (128 * 128 if lists.tiled else q_block_size * kv_block_size) * 2
 
 
 def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists, hand_over=None):
     """Backward on compacted lists -> (dq, dk, dv), bf16, shaped like q, k, v.
 
-    hand_over=True: the key-major kernel stores dS once and dQ is formed from it (fba_bwd_handover, ten products per
-    block pair); False: dQ recomputes S and dP (fba_bwd, fourteen products, no workspace); None: hand over when the
-    lists are block lists and the workspace fits DS_WORKSPACE_LIMIT_GIB and can be allocated."""
+    hand_over=True: the key-major kernel stores dS once and dQ is formed from it (fba_bwd_handover or
+    fba_bwd_tiled_handover, ten products per block pair); False: dQ recomputes S and dP (fba_bwd or fba_bwd_tiled,
+    fourteen products, no workspace); None: hand over when the workspace fits DS_WORKSPACE_LIMIT_GIB and can be
+    allocated."""
     B, Hq, Hkv, Sq, Skv = _check_qkv(q, k, v)
     _check_lists(lists, q, B, Hq, Sq, Skv, q_block_size, kv_block_size)
     if do.dtype != torch.bfloat16:
@@ -275,11 +293,9 @@ def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists,
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)
     stats = torch.empty((2, B, Hq, Sq), dtype=torch.float32, device=q.device)
-    if hand_over and lists.tiled:
-        raise ValueError("the dS hand-over works on block lists (q_block and kv_block multiples of 128)")
     pairs = ws_bytes = 0
     ds_ws = None
-    if hand_over or (hand_over is None and not lists.tiled):
+    if hand_over or hand_over is None:
         pairs, ws_bytes = ds_workspace_bytes(lists, B, Hq, q_block_size, kv_block_size)
         if ws_bytes > 0 and (hand_over or ws_bytes <= DS_WORKSPACE_LIMIT_GIB * 2 ** 30):
             try:
@@ -289,7 +305,14 @@ def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists,
                     raise
     hand_over = ds_ws is not None
     with torch.cuda.device(q.device):
-        if hand_over:
+        if hand_over and lists.tiled:
+            _lib.call(
+                "fba_bwd_tiled_handover", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), _ptr(ds_ws), ws_bytes,
+                _ptr(dq), _ptr(dk), _ptr(dv), _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx),
+                _ptr(lists.pair_base), _ptr(lists.k_slot), _ptr(lists.q_slot), pairs, lists.mask_bh,
+                B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size, _stream(),
+            )
+        elif hand_over:
             _lib.call(
                 "fba_bwd_handover", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), _ptr(ds_ws), ws_bytes,
                 _ptr(dq), _ptr(dk), _ptr(dv), _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx),

@@ -154,6 +154,29 @@ int32_t fba_bwd_tiled(const void* q, const void* k, const void* v, const void* o
                       int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
 
 /*
+ * fba_bwd_tiled with dS handed over in memory, as fba_bwd_handover does for block lists (the reference's counterpart
+ * are the reducing stores into fp32 dQ, flex_block_attn_h100.cu:707-708).  The workspace is divided into pairs of a
+ * 128-row query tile and a 128-key tile (32 KiB of bf16 dS each); only the 2 KiB units whose rows select their keys are
+ * written and read.
+ *   fba_tile_slots  numbers the listed tile pairs: pair_base [mask_bh * Skv/128 + 1] = exclusive prefix sum of the
+ *                   distinct query tiles in every kt_ent row (last entry = number of pairs in the lists), kt_slot
+ *                   [mask_bh, Skv/128, Sq/32] = pair number of every kt_ent entry (-1 beyond kt_cnt), slot_table
+ *                   [mask_bh, Sq/128, Skv/128] = pair number of (query tile, key tile), -1 where nothing is listed.
+ *                   n_qt = Sq/128, n_kt = Skv/128.
+ *   ds_ws           n_pairs * 32 KiB, 16-byte aligned; n_pairs = listed tile pairs over all (batch, head): the last
+ *                   entry of pair_base, times B * Hq when mask_bh == 1.  The caller vouches that n_pairs matches the lists.
+ * Other arguments as fba_bwd_tiled; dk, dv agree with fba_bwd_tiled's bit for bit, dq to within bf16 rounding of dS.
+ */
+int32_t fba_tile_slots(const int32_t* kt_cnt, const int32_t* kt_ent, int64_t mask_bh, int32_t n_qt, int32_t n_kt, int32_t* pair_base,
+                       int32_t* kt_slot, int32_t* slot_table, void* hip_stream);
+int32_t fba_bwd_tiled_handover(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse, float* stats,
+                               void* ds_ws, int64_t ds_ws_bytes, void* dq, void* dk, void* dv, const int32_t* qt_cnt,
+                               const int32_t* qt_ent, const int32_t* kt_cnt, const int32_t* kt_ent, const int32_t* pair_base,
+                               const int32_t* kt_slot, const int32_t* slot_table, int64_t n_pairs, int64_t mask_bh, int32_t B,
+                               int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,
+                               void* hip_stream);
+
+/*
  * Callers' side of the operator for video models.  The reference names these steps but never released them
  * (create_sta_3d_mask, create_ssta_3d_mask, create_moba_3d_mask, ssta_3d_attention: flex_block_attn/__init__.py:7-12,
  * README.md:54-55); they are specified here and checked against their own CPU restatement.

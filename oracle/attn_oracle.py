@@ -127,6 +127,39 @@ def tile_lists(block_mask, q_block, kv_block):
     return qt_cnt, qt_ent, kt_cnt, kt_ent
 
 
+def tile_pair_numbering(block_mask, q_block, kv_block):
+    """Numbers of the (128-row query tile T, 128-key tile U) pairs that hold at least one allowed (row, key), in
+    key-major order (include/fba.h, fba_tile_slots), straight from allowed(i, j) = mask[i // q_block, j // kv_block]:
+    returns (pair_base [M * n_kt + 1] with the total last, slot_table [M, n_qt, n_kt] (-1 where nothing is allowed),
+    kt_slot [M, n_kt, n_qs] = the pair number of every entry of the key-major tile list (-1 beyond its count))."""
+    m = block_mask.detach().cpu().numpy().astype(bool)
+    nQ, nK = m.shape[-2:]
+    m = m.reshape(-1, nQ, nK)
+    M, Sq, Skv = m.shape[0], nQ * q_block, nK * kv_block
+    n_qt, n_kt, n_qs = Sq // 128, Skv // 128, Sq // 32
+    pair_base = np.zeros((M * n_kt + 1,), np.int32)
+    slot_table = np.full((M, n_qt, n_kt), -1, np.int32)
+    kt_slot = np.full((M, n_kt, n_qs), -1, np.int32)
+    n = 0
+    for b in range(M):
+        for U in range(n_kt):
+            pair_base[b * n_kt + U] = n
+            cols = sorted({j // kv_block for j in range(128 * U, 128 * U + 128, 32)})
+            for T in range(n_qt):
+                rows = sorted({i // q_block for i in range(128 * T, 128 * T + 128, 16)})
+                if m[b][np.ix_(rows, cols)].any():
+                    slot_table[b, T, U] = n
+                    n += 1
+            e = 0
+            for s_ in range(n_qs):  # entries of the key-major tile list: slabs with an allowed (row, key) in this key tile
+                rows = sorted({i // q_block for i in range(32 * s_, 32 * s_ + 32, 16)})
+                if m[b][np.ix_(rows, cols)].any():
+                    kt_slot[b, U, e] = slot_table[b, s_ // 4, U]
+                    e += 1
+    pair_base[M * n_kt] = n
+    return pair_base, slot_table, kt_slot
+
+
 def block_mean(x, block):
     """(B, H, S, D) -> (B, H, S / block, D) float64 means of consecutive row blocks (include/fba.h, fba_block_mean)."""
     B, H, S, D = x.shape

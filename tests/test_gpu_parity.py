@@ -374,7 +374,7 @@ def _full_size_properties(gpu, q, k, v, do, qbs, kbs, mask, check_permutation=Tr
       * permuting key blocks together with the mask columns leaves O unchanged up to summation order."""
     import flex_block_attn_amd as fba
 
-    lists = fba.compact_block_mask(mask)
+    lists = fba.lists_for(mask, qbs, kbs)
     o1, _ = fba.forward_with_lists(q, k, torch.ones_like(v), qbs, kbs, lists)
     assert (o1.float() - 1).abs().max().item() <= 2 ** -7
     del o1
@@ -400,7 +400,7 @@ def _full_size_properties(gpu, q, k, v, do, qbs, kbs, mask, check_permutation=Tr
         perm = torch.randperm(nK, generator=torch.Generator(device="cpu").manual_seed(5)).to(gpu)
         tok = (perm[:, None] * kbs + torch.arange(kbs, device=gpu)[None, :]).reshape(-1)
         op, lsep = fba.forward_with_lists(q, k[:, :, tok].contiguous(), v[:, :, tok].contiguous(), qbs, kbs,
-                                          fba.compact_block_mask(mask[..., perm].contiguous()))
+                                          fba.lists_for(mask[..., perm].contiguous(), qbs, kbs))
         assert (op.float() - o.float()).abs().max().item() <= 2e-2 and (lsep - lse).abs().max().item() <= 1e-3
     return o, lse, dq, dk, dv
 
@@ -421,6 +421,22 @@ def test_full_size_properties(gpu):
     a = _full_size_properties(gpu, q, k, v, do, bs, bs, m, hand_over=True)
     b = _full_size_properties(gpu, q, k, v, do, bs, bs, m, check_permutation=False, hand_over=False)
     assert torch.equal(a[3], b[3]) and torch.equal(a[4], b[4])  # dK, dV: same kernel arithmetic on either path
+    assert (a[2].float() - b[2].float()).abs().max().item() <= 2e-2
+
+
+def test_fine_block_full_size_properties(gpu):
+    """Tile lists at full size: B1 H24 S30720 with independent random 64 x 64 blocks, 40 % kept, an independent mask per
+    head; the backward that hands dS over in 128 x 128 tile pairs (about 39 GB of workspace) and the recomputing one."""
+    B, H, S, bs = 1, 24, 30720, 64
+    nb = S // bs
+    q, k, v, do = _full_size_inputs(gpu, B, H, S, 21)
+    m = torch.rand((B, H, nb, nb), generator=torch.Generator().manual_seed(22)) < 0.4
+    m[..., torch.arange(nb), torch.arange(nb)] = True
+    m[..., :, 7] = False  # a key block nobody selects
+    m = m.to(gpu)
+    a = _full_size_properties(gpu, q, k, v, do, bs, bs, m, hand_over=True)
+    b = _full_size_properties(gpu, q, k, v, do, bs, bs, m, check_permutation=False, hand_over=False)
+    assert torch.equal(a[3], b[3]) and torch.equal(a[4], b[4])
     assert (a[2].float() - b[2].float()).abs().max().item() <= 2e-2
 
 
@@ -505,6 +521,22 @@ def test_pair_numbering_bit_exact(oracle, gpu):
         assert np.array_equal(q_slot.cpu().numpy(), want_slot), tuple(m.shape)
 
 
+def test_tile_pair_numbering_bit_exact(oracle, gpu):
+    """fba_tile_slots against the oracle's restatement from allowed(i, j) alone, on the tile-list cases (2-D and
+    per-(b,h) masks, empty and full masks, blocks that straddle key tiles)."""
+    import flex_block_attn_amd as fba
+    from flex_block_attn_amd import masks
+
+    for n, (qbs, kbs, nQ, nK, p) in enumerate(TILE_LIST_CASES):
+        for m in (masks.bernoulli_block_mask(nQ, nK, p, 40 + n), (torch.rand((2, 3, nQ, nK), generator=torch.Generator().manual_seed(n)) < p)):
+            lists = fba.tile_block_mask(m.to(gpu), qbs, kbs, with_pair_numbers=True)
+            want_base, want_table, want_slot = oracle.tile_pair_numbering(m, qbs, kbs)
+            for g, w, name in zip((lists.pair_base, lists.q_slot, lists.k_slot), (want_base, want_table, want_slot), ("pair_base", "slot_table", "kt_slot")):
+                assert g.dtype == torch.int32 and tuple(g.shape) == w.shape, (name, g.shape, w.shape)
+                assert np.array_equal(g.cpu().numpy(), w), f"{name} differs for q{qbs} k{kbs} mask {tuple(m.shape)}"
+            assert lists.listed_pairs() == int(want_base[-1])
+
+
 BACKWARD_PATH_CASES = [
     # B, Hq, Hkv, Sq, Skv, q_block, kv_block, mask dims, density
     (1, 2, 2, 1536, 1536, 384, 384, 4, 0.5),
@@ -513,14 +545,22 @@ BACKWARD_PATH_CASES = [
     (1, 2, 1, 1024, 768, 256, 128, 4, 0.4),    # q block larger than the kv block
     (1, 6, 2, 768, 1152, 384, 128, 2, 0.7),
     (2, 2, 2, 384, 384, 128, 384, 4, 1.0),
+    # tile lists: dS travels in 128 x 128 tile pairs, only the 32 x 32 units that some row selects
+    (1, 2, 2, 512, 512, 64, 64, 4, 0.5),
+    (1, 3, 3, 768, 768, 16, 64, 2, 0.4),       # one 2-D mask for three heads
+    (2, 4, 2, 512, 768, 32, 192, 4, 0.5),      # grouped kv heads; key blocks that straddle key tiles
+    (1, 2, 1, 1152, 1152, 48, 192, 4, 0.4),
+    (1, 2, 2, 768, 768, 128, 64, 4, 0.5),
+    (1, 2, 2, 512, 768, 64, 128, 4, 0.3),
+    (1, 2, 2, 256, 256, 64, 64, 4, 1.0),
 ]
 
 
 @pytest.mark.parametrize("hand_over", [False, True], ids=["recompute", "handover"])
 @pytest.mark.parametrize("cfg", BACKWARD_PATH_CASES, ids=lambda c: "B%d_Hq%d_Hkv%d_Sq%d_Skv%d_q%d_k%d_m%d_p%s" % c)
 def test_both_backward_paths_against_oracle(oracle, gpu, cfg, hand_over):
-    """fba_bwd (dQ recomputes S and dP) and fba_bwd_handover (dQ from the dS the key-major kernel stored), each against
-    the C oracle; masks with an empty query block and an unselected key block."""
+    """fba_bwd / fba_bwd_tiled (dQ recomputes S and dP) and fba_bwd_handover / fba_bwd_tiled_handover (dQ from the dS the
+    key-major kernel stored), each against the C oracle; masks with an empty query block and an unselected key block."""
     import flex_block_attn_amd as fba
 
     B, Hq, Hkv, Sq, Skv, qbs, kbs, mdim, density = cfg
@@ -536,7 +576,7 @@ def test_both_backward_paths_against_oracle(oracle, gpu, cfg, hand_over):
     o_ref, lse_ref = oracle.c_attention_forward(qb, kb, vb, m, qbs, kbs)
     g_ref = oracle.c_attention_backward(qb, kb, vb, o_ref, lse_ref, dob, m, qbs, kbs)
     qg, kg, vg, dog = (t.to(gpu) for t in (qb, kb, vb, dob))
-    lists = fba.compact_block_mask(m.to(gpu))
+    lists = fba.lists_for(m.to(gpu), qbs, kbs)
     o, lse = fba.forward_with_lists(qg, kg, vg, qbs, kbs, lists)
     print(f"backward path hand_over={hand_over} cfg={cfg}", flush=True)
     grads = fba.backward_with_lists(qg, kg, vg, o, lse, dog, qbs, kbs, lists, hand_over=hand_over)
@@ -567,6 +607,16 @@ def test_backward_falls_back_without_workspace(gpu, monkeypatch):
     empty = fba.compact_block_mask(torch.zeros((6, 6), dtype=torch.bool, device=gpu))
     o0, lse0 = fba.forward_with_lists(q, k, v, 128, 128, empty)
     for t in fba.backward_with_lists(q, k, v, o0, lse0, do, 128, 128, empty, hand_over=True):
+        assert t.abs().max().item() == 0.0
+    # the same with tile lists
+    tl = fba.tile_block_mask(masks.bernoulli_block_mask(12, 12, 0.5, 2).to(gpu), 64, 64)
+    o, lse = fba.forward_with_lists(q, k, v, 64, 64, tl)
+    want = fba.backward_with_lists(q, k, v, o, lse, do, 64, 64, tl, hand_over=False)
+    for a, b in zip(fba.backward_with_lists(q, k, v, o, lse, do, 64, 64, tl), want):
+        assert torch.equal(a, b)
+    empty = fba.tile_block_mask(torch.zeros((12, 12), dtype=torch.bool, device=gpu), 64, 64)
+    o0, lse0 = fba.forward_with_lists(q, k, v, 64, 64, empty)
+    for t in fba.backward_with_lists(q, k, v, o0, lse0, do, 64, 64, empty, hand_over=True):
         assert t.abs().max().item() == 0.0
 
 

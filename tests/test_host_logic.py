@@ -75,6 +75,15 @@ def test_c_abi_argument_validation(lib):
     assert h.fba_tile_lists(f, 1, 4, 4, 24, 64, f, f, f, f, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_tile_lists(f, 1, 4, 4, 64, 64, f, _null(), f, f, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_bwd_tiled(*([f] * 14), 1, 1, 2, 2, 256, 256, 128, 64, 96, _null()) == lib.FBA_ERR_INVALID
+    # tile-pair numbering and the tile-list backward that hands dS over
+    assert h.fba_tile_slots(f, f, 0, 2, 2, f, f, f, _null()) == lib.FBA_ERR_INVALID and b"positive" in h.fba_last_error()
+    assert h.fba_tile_slots(f, f, 1, 2, 2, f, _null(), f, _null()) == lib.FBA_ERR_INVALID
+    tho = [f] * 8 + [2 * 32768] + [f] * 10
+    assert h.fba_bwd_tiled_handover(*tho, 3, 1, 1, 2, 2, 256, 256, 128, 64, 64, _null()) == lib.FBA_ERR_INVALID
+    assert b"3 tile pairs" in h.fba_last_error()
+    assert h.fba_bwd_tiled_handover(*tho, 2, 1, 1, 2, 2, 192, 192, 128, 64, 64, _null()) == lib.FBA_ERR_UNSUPPORTED
+    tho[18] = _null()  # slot_table
+    assert h.fba_bwd_tiled_handover(*tho, 2, 1, 1, 2, 2, 256, 256, 128, 64, 64, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_mask_compact(f, 0, 4, 4, f, f, f, f, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_mask_compact(_null(), 1, 4, 4, f, f, f, f, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_bwd_stats(f, f, f, f, 16, 64, _null()) == lib.FBA_ERR_INVALID
@@ -296,6 +305,12 @@ def test_block_lists_are_validated_before_any_launch():
     _check_lists(tiled, q, 1, 2, 256, 256, 64, 64)
     tiled.k_idx = torch.zeros((1, 2, 4), **i32)
     with pytest.raises(ValueError, match="k_idx"):
+        _check_lists(tiled, q, 1, 2, 256, 256, 64, 64)
+    tiled.k_idx = torch.zeros((1, 2, 8), **i32)
+    tiled.pair_base, tiled.q_slot, tiled.k_slot = torch.zeros((3,), **i32), torch.zeros((1, 2, 2), **i32), torch.zeros((1, 2, 8), **i32)
+    _check_lists(tiled, q, 1, 2, 256, 256, 64, 64)
+    tiled.k_slot = torch.zeros((1, 2, 4), **i32)
+    with pytest.raises(ValueError, match="k_slot"):
         _check_lists(tiled, q, 1, 2, 256, 256, 64, 64)
 
 

@@ -322,6 +322,36 @@ def test_pair_numbering(oracle):
         assert sorted(seen) == list(range(int(m.sum())))
 
 
+def test_tile_pair_numbering(oracle):
+    """oracle.tile_pair_numbering against the token-level mask: a (query tile, key tile) pair is numbered exactly when
+    the dense mask (numpy's kron) has an allowed element inside that 128 x 128 square, the numbers run 0..n-1 in
+    key-major order, and every entry of the key-major tile list carries the number of the square its slab lies in."""
+    for shape, qb, kb, p, seed in (((8, 4), 32, 64, 0.3, 0), ((2, 2, 16, 2), 16, 192, 0.2, 1), ((4, 4), 64, 64, 0.0, 2),
+                                   ((1, 2, 8, 6), 48, 64, 0.5, 3), ((2, 4), 128, 64, 1.0, 4)):
+        m = torch.rand(shape, generator=torch.Generator().manual_seed(seed)) < p
+        nQ, nK = shape[-2:]
+        Sq, Skv = nQ * qb, nK * kb
+        if Sq % 128 or Skv % 128:
+            continue
+        n_qt, n_kt = Sq // 128, Skv // 128
+        pair_base, table, kt_slot = oracle.tile_pair_numbering(m, qb, kb)
+        dense = np.kron(m.numpy().reshape(-1, nQ, nK), np.ones((qb, kb), bool))
+        M = dense.shape[0]
+        squares = dense.reshape(M, n_qt, 128, n_kt, 128).any(axis=(2, 4))  # [M, T, U]
+        assert np.array_equal(table >= 0, squares)
+        order = [table[b, T, U] for b in range(M) for U in range(n_kt) for T in range(n_qt) if squares[b, T, U]]
+        assert order == list(range(len(order))) and pair_base[-1] == len(order)
+        assert np.array_equal(pair_base[:-1], np.concatenate([[0], np.cumsum(squares.transpose(0, 2, 1).reshape(-1, n_qt).sum(1))[:-1]]))
+        _, _, kt_cnt, kt_ent = oracle.tile_lists(m, qb, kb)
+        for b in range(M):
+            for U in range(n_kt):
+                for e in range(kt_ent.shape[2]):
+                    if e < kt_cnt[b, U]:
+                        assert kt_slot[b, U, e] == table[b, (kt_ent[b, U, e] >> 8) // 4, U] >= 0
+                    else:
+                        assert kt_slot[b, U, e] == -1
+
+
 def test_sliding_tile_mask_restatement(oracle):
     """Pins oracle.sta_window / sta_3d_mask / sta_token_mask: hand-computed windows, a hand-listed row of an asymmetric
     grid, the Kronecker product of 1-D band matrices (numpy's kron fixes the T-major, W-minor enumeration: swapping two
