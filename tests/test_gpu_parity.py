@@ -354,15 +354,16 @@ def test_deterministic(gpu):
 
     g = torch.Generator(device="cpu").manual_seed(9)
     q, k, v, do = (torch.randn((1, 3, 1536, 128), generator=g).to(torch.bfloat16).to(gpu) for _ in range(4))
-    m = masks.random_block_mask(1, 3, 4, 4, 2, 10).to(gpu)
-    outs = []
-    for _ in range(2):
-        qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
-        o = fba.flex_block_attn_func(qq, kk, vv, 384, 384, m)
-        o.backward(do)
-        outs.append((o.detach(), qq.grad, kk.grad, vv.grad))
-    for a, b in zip(*outs):
-        assert torch.equal(a, b)
+    # block lists, then tile lists (64-row blocks): forward and the dS hand-over of backward write every element once
+    for bs, m in ((384, masks.random_block_mask(1, 3, 4, 4, 2, 10)), (64, masks.random_block_mask(1, 3, 24, 24, 9, 11))):
+        outs = []
+        for _ in range(2):
+            qq, kk, vv = (t.clone().requires_grad_(True) for t in (q, k, v))
+            o = fba.flex_block_attn_func(qq, kk, vv, bs, bs, m.to(gpu))
+            o.backward(do)
+            outs.append((o.detach(), qq.grad, kk.grad, vv.grad))
+        for a, b in zip(*outs):
+            assert torch.equal(a, b)
 
 
 def _full_size_properties(gpu, q, k, v, do, qbs, kbs, mask, check_permutation=True, hand_over=None):
