@@ -2,7 +2,7 @@
 //
 // One work-group of 4 waves owns 128 consecutive query rows of one (batch, head); wave w owns rows [32w, 32w+32).
 // The work-group walks the active-key-block list of its query block and streams every selected key block through
-// LDS as 64-key slabs of K and V (two buffers each).
+// LDS as 32-key slabs of K and V (a ring of four 8 KiB buffers each).
 //
 // Everything is kept "transposed" so that softmax statistics are per-lane scalars (lane = query row):
 //   S^T[key, q]  = K[key, :] . Q[q, :]            A = K slab rows from LDS (128-bit fetches), B = Q in registers

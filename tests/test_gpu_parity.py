@@ -680,3 +680,28 @@ def test_matrix_pipe_probe(gpu):
     _lib.call("fba_probe_mfma", _ptr(src), _ptr(sink), 4, 10, _stream())
     # each MFMA adds 16 * 0.25 = 4 to every element; 10 of them per accumulator, 4 accumulators x 16 elements summed
     assert torch.equal(sink, torch.full_like(sink, 4.0 * 10 * 64))
+
+
+@pytest.mark.parametrize("block_size", [64, 128, 384])
+def test_readme_usage_verbatim(oracle, gpu, block_size):
+    """The reference README's usage section (README.md:24-53), run as written: its two imports, a list-of-lists
+    `selected_blocks`, `create_sparse_mask`, the call; on a (block_size * 2) x (block_size * 2) problem as there, at the
+    block sizes it names.  The result is compared with the oracle under that 2 x 2 mask."""
+    from flex_block_attn import flex_block_attn_func
+    from benchmark.utils.utils import create_sparse_mask
+
+    g = torch.Generator(device="cpu").manual_seed(block_size)
+    q, key, value = (torch.randn((1, 2, block_size * 2, 128), generator=g).to(torch.bfloat16).to(gpu) for _ in range(3))
+    query = q
+    q_block_size = k_block_size = block_size
+    # take a (block_size * 2)*(block_size * 2) as an example
+    selected_blocks = [[0, 1], [1, 0]]
+    # create block mask with selected blocks
+    sparse_mask = create_sparse_mask(q, block_size, selected_blocks)
+    block_mask = sparse_mask
+    # compute
+    output = flex_block_attn_func(query, key, value, q_block_size, k_block_size, block_mask)
+
+    assert sparse_mask.dtype == torch.bool and sparse_mask.cpu().tolist() == [[False, True], [True, False]]
+    want, _ = oracle.c_attention_forward(query.cpu(), key.cpu(), value.cpu(), sparse_mask.cpu(), block_size, block_size)
+    _check(oracle, output, want, "o", {})
