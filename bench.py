@@ -187,6 +187,8 @@ def main():
     ap.add_argument("--recompute", action="store_true", help="backward without the dS workspace (fba_bwd: dQ recomputes S and dP)")
     ap.add_argument("--inputs", choices=["random", "zeros"], default="random",
                     help="zeros: all-zero q, k, v, dO (a probe of the power limit, not a benchmark figure)")
+    ap.add_argument("--fwd-tile-rows", choices=["128", "384"], default=None,
+                    help="query rows per forward work-group where both kernels apply (measurement of the two forward variants)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy three times, as the known-size yardstick for rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--probe-atomics", action="store_true",
@@ -195,6 +197,8 @@ def main():
     args = ap.parse_args()
     if args.probe_atomics:
         return probe_atomics()
+    if args.fwd_tile_rows:
+        os.environ["FBA_FWD_TILE_ROWS"] = args.fwd_tile_rows
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU only: every box in this build has a single MI355X (use --gpus 1)")
     if not torch.cuda.is_available():

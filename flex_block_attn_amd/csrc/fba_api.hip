@@ -1,6 +1,7 @@
 // C ABI entry points: argument validation, variant selection, launches.  See include/fba.h for the contract.
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <mutex>
 
@@ -103,6 +104,10 @@ int fwd_impl(const void* q, const void* k, const void* v, void* o, float* lse, c
   p.q_block = q_block; p.k_block = k_block;
   p.scale_log2e = 1.4426950408889634f / 11.313708498984761f;
   p.tiled = tiled ? 1 : 0;
+  {
+    const char* rows = getenv("FBA_FWD_TILE_ROWS");
+    p.variant = rows && atoi(rows) == 384 ? 0 : 1;  // 128-row work-groups unless asked otherwise
+  }
   hipError_t e = fba::launch_fwd(p, (hipStream_t)hip_stream);
   return e == hipSuccess ? FBA_OK : hip_fail(e, "forward launch");
 }

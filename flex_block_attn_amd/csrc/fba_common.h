@@ -201,6 +201,62 @@ struct SlabDma {
   }
 };
 
+// The same copy for the two slabs (K, V) a step of a query-major kernel brings in, by the kWaves waves of its work-group.
+// A wave-level copy fills 4 rows; a slab is eight of them.  kWaves = 4: wave w copies rows 8w .. 8w+7 of both slabs.
+// kWaves = 12: rows 4w .. 4w+3 of the K slab by waves 0..7, rows 4(w-4) .. of the V slab by waves 4..11, so waves 4..7
+// issue two copies per step and the others one.
+template <int kWaves>
+struct SlabDmaShared {
+  static_assert(kWaves == 4 || kWaves == 12, "4 or 12 waves");
+  uint32_t off[2];  // kWaves = 4: the wave's two row groups; kWaves = 12: its row group in the K slab, in the V slab
+  uint32_t dst[2];
+  bool has_k, has_v;
+  FBA_DEVICE static uint32_t lane_off(int row_group, int lane) {
+    const int row = 4 * row_group + (lane >> 4);
+    return (uint32_t)(row * kRowBytes + (((lane & 15) ^ swz(row)) << 4));
+  }
+  FBA_DEVICE void init(int wave, int lane) {
+    if constexpr (kWaves == 4) {
+      has_k = has_v = true;
+      off[0] = lane_off(2 * wave, lane);
+      off[1] = lane_off(2 * wave + 1, lane);
+      dst[0] = (uint32_t)(2 * wave * 4 * kRowBytes);
+      dst[1] = dst[0] + 4 * kRowBytes;
+    } else {
+      has_k = wave < 8;
+      has_v = wave >= 4;
+      const int gk = wave & 7, gv = (wave - 4) & 7;
+      off[0] = lane_off(gk, lane);
+      off[1] = lane_off(gv, lane);
+      dst[0] = (uint32_t)(gk * 4 * kRowBytes);
+      dst[1] = (uint32_t)(gv * 4 * kRowBytes);
+    }
+  }
+  FBA_DEVICE void copy_k(uint32_t slab_lds, const char* src) const {
+    if constexpr (kWaves == 4) {
+      dma16(slab_lds + dst[0], src, off[0]);
+      dma16(slab_lds + dst[1], src, off[1]);
+    } else {
+      if (has_k) dma16(slab_lds + dst[0], src, off[0]);
+    }
+  }
+  FBA_DEVICE void copy_v(uint32_t slab_lds, const char* src) const {
+    if constexpr (kWaves == 4) {
+      copy_k(slab_lds, src);
+    } else {
+      if (has_v) dma16(slab_lds + dst[1], src, off[1]);
+    }
+  }
+  // Wait until only the copies this wave issued during the last two steps (one K and one V request each) may be in flight.
+  FBA_DEVICE void wait_two_steps() const {
+    if constexpr (kWaves == 4) {
+      wait_vmem<8>();
+    } else {
+      if (has_k && has_v) wait_vmem<4>(); else wait_vmem<2>();
+    }
+  }
+};
+
 // Per-lane LDS offsets for row-major A/B operand fetches of a 32-row slab: rd[ks] addresses row (lane % 32),
 // chunk 2*ks + lane/32.  Add 32*kRowBytes per further slab (rows stay congruent mod 16, so swz is unchanged).
 struct RowMajorOffsets {

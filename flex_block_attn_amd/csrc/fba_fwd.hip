@@ -113,10 +113,15 @@ FBA_DEVICE void softmax_exp(FwdState& st, f32x16& s, bf16x8 (&pk)[2], bool activ
 
 // kTiled = false: q_block is a multiple of 128, the list of a work-group is the block list of its query block.
 // kTiled = true: tile lists with a predicate per 16-row group (any q_block that is a multiple of 16).
-template <bool kTiled>
-__global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_per_eu(2, 2))) void fwd_kernel(const FwdParams p) {
+// kWaves = 4: 128 query rows per work-group, two work-groups per CU.  kWaves = 12 (q_block a multiple of 384, block
+// lists): 384 rows, one work-group per CU with three waves per SIMD; every K / V slab brought into LDS then feeds three
+// times as many matrix instructions (the reference shares its K / V tiles between three consumer groups for the same
+// reason, flex_block_attn_h100.cu:912-928).
+template <bool kTiled, int kWaves>
+__global__ __attribute__((amdgpu_flat_work_group_size(64 * kWaves, 64 * kWaves), amdgpu_waves_per_eu(kWaves == 12 ? 3 : 2, kWaves == 12 ? 3 : 2))) void fwd_kernel(const FwdParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];  // K ring [4][8 KiB] | V ring [4][8 KiB]
-  constexpr int TQ = 128;
+  constexpr int TQ = 32 * kWaves;
+  static_assert(!kTiled || kWaves == 4, "tile lists describe 128-row tiles");
 
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -156,7 +161,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 #pragma unroll
     for (int r = 0; r < 16; ++r) st.acc_o[mb][r] = 0.f;
 
-  SlabDma dma;
+  SlabDmaShared<kWaves> dma;
   dma.init(wave, lane);
   char* const k_lds = smem;
   char* const v_lds = smem + kRing * kSlabBytes;
@@ -181,7 +186,9 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     }
     return off;
   };
-  auto copy_slab = [&](uint32_t dst, const char* src) { dma.copy(dst, src); };
+  // K slabs and V slabs are brought in by different (overlapping, for 12 waves) sets of waves
+  auto copy_k = [&](uint32_t dst, const char* src) { dma.copy_k(dst, src); };
+  auto copy_v = [&](uint32_t dst, const char* src) { dma.copy_v(dst, src); };
 
   if (nsteps > 0) {
     // prologue: K_0..K_3 and V_0..V_2 requested, S_0 computed, then K_4 into the buffer of K_0
@@ -190,11 +197,11 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     for (int j = 0; j < 4; ++j)
       if (j < nsteps) {
         off[j] = next_off();
-        copy_slab(k_dst + j * kSlabBytes, kp + off[j]);
+        copy_k(k_dst + j * kSlabBytes, kp + off[j]);
       }
 #pragma unroll
     for (int j = 0; j < 3; ++j)
-      if (j < nsteps) copy_slab(v_dst + j * kSlabBytes, vp + off[j]);
+      if (j < nsteps) copy_v(v_dst + j * kSlabBytes, vp + off[j]);
     wait_vmem<0>();
     __syncthreads();
 #pragma unroll
@@ -204,7 +211,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     __syncthreads();
     if (4 < nsteps) {
       off[4] = next_off();
-      copy_slab(k_dst, kp + off[4]);
+      copy_k(k_dst, kp + off[4]);
     }
     int64_t hist0 = off[4], hist1 = off[3];  // offsets of the two youngest K requests
 
@@ -248,16 +255,16 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
       pin(p_prev[0]);
       pin(p_prev[1]);
       s_cur = s_nxt;
-      // K_{t+2} and V_t must have landed; the copies requested after steps t-2 and t-1 (4 each) may still fly
-      if (t + 5 < nsteps) wait_vmem<8>(); else wait_vmem<0>();
+      // K_{t+2} and V_t must have landed; the copies this wave requested after steps t-2 and t-1 may still fly
+      if (t + 5 < nsteps) dma.wait_two_steps(); else wait_vmem<0>();
       __syncthreads();
       const int64_t v_off = hist1;
       hist1 = hist0;
       if (t + 5 < nsteps) {
         hist0 = next_off();
-        copy_slab(k_dst + ((R + 1) & 3) * kSlabBytes, kp + hist0);
+        copy_k(k_dst + ((R + 1) & 3) * kSlabBytes, kp + hist0);
       }
-      if (t + 3 < nsteps) copy_slab(v_dst + ((R + 3) & 3) * kSlabBytes, vp + v_off);
+      if (t + 3 < nsteps) copy_v(v_dst + ((R + 3) & 3) * kSlabBytes, vp + v_off);
     };
     step(IC<0>{}, std::true_type{}, 0);
     step(IC<1>{}, std::false_type{}, 1);
@@ -289,15 +296,14 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 
 hipError_t launch_fwd(FwdParams p, hipStream_t stream) {
   constexpr int kSmem = 2 * kRing * kSlabBytes;
-  p.num_items = p.B * p.Hq * (p.Sq / 128);
+  const bool wide = !p.tiled && p.q_block % 384 == 0 && p.variant != 1;
+  void (*fn)(const FwdParams) = p.tiled ? &fwd_kernel<true, 4> : wide ? &fwd_kernel<false, 12> : &fwd_kernel<false, 4>;
+  const int rows = wide ? 384 : 128;
+  p.num_items = p.B * p.Hq * (p.Sq / rows);
   p.items_per_xcd = (p.num_items + kNumXcd - 1) / kNumXcd;
-  const void* fn = p.tiled ? reinterpret_cast<const void*>(&fwd_kernel<true>) : reinterpret_cast<const void*>(&fwd_kernel<false>);
-  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
   if (e != hipSuccess) return e;
-  if (p.tiled)
-    hipLaunchKernelGGL(fwd_kernel<true>, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
-  else
-    hipLaunchKernelGGL(fwd_kernel<false>, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
+  hipLaunchKernelGGL(fn, dim3(p.items_per_xcd * kNumXcd), dim3(rows * 2), kSmem, stream, p);
   return hipGetLastError();
 }
 

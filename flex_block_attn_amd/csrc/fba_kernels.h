@@ -11,6 +11,25 @@ namespace fba {
 //   k_cnt [mask_bh, nK], k_idx [mask_bh, nK, nQ]: for every key block the ascending query blocks that select it.
 // mask_bh is B*Hq, or 1 when one 2-D mask is shared by every (batch, head).
 
+// Tail splitting.  Work-groups are handed to free slots in index order, so the last (items % slots) items of a launch
+// would run as a partial round with most compute units idle.  With a workspace, those items are cut into `parts` ranges of
+// their lists, each run by its own work-group at the end of the grid; the work-groups store fp32 partial results into the
+// workspace and a small merge kernel combines them in a fixed order.  Items [0, first) run whole.
+struct SplitPlan {
+  float* ws;      // null: nothing is split
+  int first;      // first item that is split
+  int parts;      // work-groups per split item (>= 2 when ws is set)
+  int main_wgs;   // work-groups in front of the split ones (a multiple of the XCD count)
+};
+
+// Items and work-group slots of a launch -> plan.  `slot_bytes` is what one part stores; the workspace must hold
+// (items - first) * parts of them.
+SplitPlan plan_split(int num_items, int wgs_per_cu, int64_t slot_bytes, void* ws, int64_t ws_bytes);
+
+constexpr int kSplitMaxSlots = 512;                           // two work-groups on each of 256 compute units
+constexpr int64_t kSplitSlotBytes = 128 * 128 * 4 * 2;        // dK and dV partials of a key tile; forward: O^T + (m, l)
+constexpr int64_t kSplitWsBytes = (kSplitMaxSlots / 2) * kSplitSlotBytes + (1 << 20);
+
 struct FwdParams {
   const __bf16* q;
   const __bf16* k;
@@ -26,6 +45,8 @@ struct FwdParams {
   // tiled = 1: q_cnt / q_idx are tile lists (qt_cnt [mask_bh, Sq/128], qt_ent [mask_bh, Sq/128, nK], see
   // tile_lists_kernel) instead of block lists
   int tiled;
+  int variant;  // 0: 384-row work-groups where q_block allows (measurement of that variant); 1: 128-row work-groups
+  SplitPlan split;
 };
 
 struct BwdParams {
@@ -65,6 +86,7 @@ struct BwdParams {
   const int32_t* q_slot;
   const int32_t* k_slot;
   const char* zero_unit;
+  SplitPlan split;
 };
 
 hipError_t launch_mask_compact(const uint8_t* mask, int64_t mask_bh, int nQ, int nK, int32_t* q_cnt, int32_t* q_idx,
