@@ -189,6 +189,9 @@ def main():
                     help="zeros: all-zero q, k, v, dO (a probe of the power limit, not a benchmark figure)")
     ap.add_argument("--fwd-tile-rows", choices=["128", "384"], default=None,
                     help="query rows per forward work-group where both kernels apply (measurement of the two forward variants)")
+    ap.add_argument("--dkdv-keys-per-wave", choices=["32", "64"], default=None,
+                    help="keys per wave of the dK/dV kernel on block lists: 32 (two waves per SIMD, the default) or 64 (one wave per "
+                         "SIMD, accumulators in accumulation registers); measurement of the two variants")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 256 MiB device copy three times, as the known-size yardstick for rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     ap.add_argument("--probe-atomics", action="store_true",
@@ -199,6 +202,8 @@ def main():
         return probe_atomics()
     if args.fwd_tile_rows:
         os.environ["FBA_FWD_TILE_ROWS"] = args.fwd_tile_rows
+    if args.dkdv_keys_per_wave:
+        os.environ["FBA_DKDV_KEYS_PER_WAVE"] = args.dkdv_keys_per_wave
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU only: every box in this build has a single MI355X (use --gpus 1)")
     if not torch.cuda.is_available():
@@ -244,11 +249,12 @@ def main():
     stats = torch.empty((2, B, H, S), dtype=torch.float32, device=dev)
     o2, lse2 = torch.empty_like(o), torch.empty_like(lse)
     common = (lists.mask_bh, B, H, H, S, S, D, qbs, kbs)
+    _sp, sp_ptr, sp_bytes = interface._split_workspace(dev)  # tail-splitting workspace, as the operator passes it
     kernels = {
         "mask_compact": lambda: _lib.call("fba_mask_compact", _ptr(mask), lists.mask_bh, lists.nQ, lists.nK, _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), _stream()),
-        "fwd": lambda: _lib.call("fba_fwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o2), _ptr(lse2), _ptr(lists.q_cnt), _ptr(lists.q_idx), *common, _stream()),
+        "fwd": lambda: _lib.call("fba_fwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o2), _ptr(lse2), _ptr(lists.q_cnt), _ptr(lists.q_idx), *common, sp_ptr, sp_bytes, _stream()),
         "bwd_stats": lambda: _lib.call("fba_bwd_stats", _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), B * H * S, D, _stream()),
-        "bwd_dkdv": lambda: _lib.call("fba_bwd_dkdv", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(stats), _ptr(dk), _ptr(dv), _ptr(lists.k_cnt), _ptr(lists.k_idx), *common, _stream()),
+        "bwd_dkdv": lambda: _lib.call("fba_bwd_dkdv", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(stats), _ptr(dk), _ptr(dv), _ptr(lists.k_cnt), _ptr(lists.k_idx), *common, sp_ptr, sp_bytes, _stream()),
         "bwd_dq": lambda: _lib.call("fba_bwd_dq", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(stats), _ptr(dq), _ptr(lists.q_cnt), _ptr(lists.q_idx), *common, _stream()),
     }
     if mask_fn:
@@ -257,14 +263,15 @@ def main():
         kernels["block_mean_q"] = lambda: _lib.call("fba_block_mean", _ptr(q), _ptr(q_mean), B * H, S, qbs, D, _stream())
         kernels["block_mean_k"] = lambda: _lib.call("fba_block_mean", _ptr(k), _ptr(k_mean), B * H, S, kbs, D, _stream())
         kernels["ssta_mask"] = lambda: _lib.call("fba_ssta_mask", _ptr(q_mean), _ptr(k_mean), None, _ptr(mask2), B, H, H, S // qbs, S // kbs, qbs, kbs, 16, 1, 1, _stream())
-    # the hand-over backward (what the step uses when its workspace fits): dK/dV + dS store, then dQ from the stored dS
+    # the hand-over backward: dK/dV + dS store, then dQ from the stored dS.  The step runs it in chunks of heads through a
+    # bounded workspace; the two kernels are timed here on all heads at once (one workspace for everything)
     pairs, ws_bytes = interface.ds_workspace_bytes(lists, B, H, qbs, kbs)
-    hand_over = 0 < ws_bytes <= interface.DS_WORKSPACE_LIMIT_GIB * 2 ** 30 and not args.recompute
+    hand_over = 0 < ws_bytes <= 64 * 2 ** 30 and not args.recompute
     if hand_over:
         ds_ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
         ho = (pairs, lists.mask_bh, B, H, H, S, S, D, qbs, kbs)
-        kernels["bwd_dkdv_handover"] = lambda: _lib.call("fba_bwd_dkdv_handover", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(stats), _ptr(dk), _ptr(dv), _ptr(ds_ws), ws_bytes, _ptr(lists.k_cnt), _ptr(lists.k_idx), _ptr(lists.pair_base), *ho, _stream())
-        kernels["bwd_dq_from_ds"] = lambda: _lib.call("fba_bwd_dq_from_ds", _ptr(k), _ptr(ds_ws), ws_bytes, _ptr(dq), _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.q_slot), _ptr(lists.pair_base), *ho, _stream())
+        kernels["bwd_dkdv_handover"] = lambda: _lib.call("fba_bwd_dkdv_handover", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(stats), _ptr(dk), _ptr(dv), _ptr(ds_ws), ws_bytes, _ptr(lists.k_cnt), _ptr(lists.k_idx), _ptr(lists.pair_base), *ho, sp_ptr, sp_bytes, _stream())
+        kernels["bwd_dq_from_ds"] = lambda: _lib.call("fba_bwd_dq_from_ds", _ptr(k), _ptr(ds_ws), ws_bytes, _ptr(dq), _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.q_slot), _ptr(lists.pair_base), *ho, sp_ptr, sp_bytes, _stream())
         kernels["pair_slots"] = lambda: _lib.call("fba_pair_slots", _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), lists.mask_bh, lists.nQ, lists.nK, _ptr(lists.pair_base), _ptr(lists.q_slot), _stream())
     iters = max(5, args.steps)
     kms = {}

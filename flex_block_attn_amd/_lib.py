@@ -23,13 +23,14 @@ SIGNATURES = {
     "fba_version": (_c_i32, []),
     "fba_last_error": (ctypes.c_char_p, []),
     "fba_mask_compact": (_c_i32, [_c_ptr, _c_i64, _c_i32, _c_i32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr]),
-    "fba_fwd": (_c_i32, [_c_ptr] * 7 + [_c_i64] + [_c_i32] * 8 + [_c_ptr]),
-    "fba_bwd": (_c_i32, [_c_ptr] * 14 + [_c_i64] + [_c_i32] * 8 + [_c_ptr]),
+    "fba_split_workspace_bytes": (_c_i64, []),
+    "fba_fwd": (_c_i32, [_c_ptr] * 7 + [_c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
+    "fba_bwd": (_c_i32, [_c_ptr] * 14 + [_c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
     "fba_probe_mfma": (_c_i32, [_c_ptr, _c_ptr, _c_i32, _c_i32, _c_ptr]),
     "fba_pair_slots": (_c_i32, [_c_ptr] * 4 + [_c_i64, _c_i32, _c_i32, _c_ptr, _c_ptr, _c_ptr]),
-    "fba_bwd_handover": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_ptr] * 9 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr]),
-    "fba_bwd_dkdv_handover": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_ptr] * 3 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr]),
-    "fba_bwd_dq_from_ds": (_c_i32, [_c_ptr] * 2 + [_c_i64] + [_c_ptr] * 5 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr]),
+    "fba_bwd_handover": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_ptr] * 9 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
+    "fba_bwd_dkdv_handover": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_ptr] * 3 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
+    "fba_bwd_dq_from_ds": (_c_i32, [_c_ptr] * 2 + [_c_i64] + [_c_ptr] * 5 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
     "fba_tile_slots": (_c_i32, [_c_ptr, _c_ptr, _c_i64, _c_i32, _c_i32, _c_ptr, _c_ptr, _c_ptr, _c_ptr]),
     "fba_bwd_tiled_handover": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_ptr] * 10 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr]),
     "fba_bwd_noalloc": (_c_i32, [_c_ptr] * 13 + [_c_i64] + [_c_i32] * 8 + [_c_ptr]),
@@ -41,7 +42,7 @@ SIGNATURES = {
     "fba_bwd_tiled": (_c_i32, [_c_ptr] * 14 + [_c_i64] + [_c_i32] * 8 + [_c_ptr]),
     "fba_bwd_stats": (_c_i32, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i32, _c_ptr]),
     "fba_bwd_dq": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_i32] * 8 + [_c_ptr]),
-    "fba_bwd_dkdv": (_c_i32, [_c_ptr] * 9 + [_c_i64] + [_c_i32] * 8 + [_c_ptr]),
+    "fba_bwd_dkdv": (_c_i32, [_c_ptr] * 9 + [_c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
 }
 
 _lib = None

@@ -15,7 +15,7 @@ import sys
 CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 LIB_NAME = "libfba_gfx950.so"
 LIB_PATH = os.path.join(CSRC, LIB_NAME)
-SOURCES = ["fba_api.hip", "fba_mask_compact.hip", "fba_ssta_mask.hip", "fba_fwd.hip", "fba_bwd_dq.hip", "fba_bwd_dq_ds.hip", "fba_bwd_dkdv.hip", "fba_probe.hip"]
+SOURCES = ["fba_api.hip", "fba_mask_compact.hip", "fba_ssta_mask.hip", "fba_fwd.hip", "fba_bwd_dq.hip", "fba_bwd_dq_ds.hip", "fba_bwd_dkdv.hip", "fba_bwd_dkdv64.hip", "fba_probe.hip", "fba_split.hip"]
 
 # Per-file extras.  --amdgpu-mfma-vgpr-form keeps MFMA accumulators in ordinary VGPRs, so the softmax arithmetic on
 # them needs no accumulator-register copies; it pays off where the whole working set fits 256 registers.
@@ -23,6 +23,7 @@ EXTRA_FLAGS = {
     "fba_fwd.hip": ["-mllvm", "--amdgpu-mfma-vgpr-form"],
     "fba_bwd_dq.hip": ["-mllvm", "--amdgpu-mfma-vgpr-form"],
     "fba_bwd_dq_ds.hip": ["-mllvm", "--amdgpu-mfma-vgpr-form"],
+    "fba_bwd_dkdv64.hip": ["-mllvm", "--amdgpu-mfma-vgpr-form"],
 }
 
 # -packed-fp32-ops is switched off: hipcc otherwise fuses pairs of fp32 operations into packed instructions.

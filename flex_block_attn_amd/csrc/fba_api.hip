@@ -54,7 +54,23 @@ int check_ptrs(std::initializer_list<std::pair<const char*, const void*>> ps) {
   return FBA_OK;
 }
 
+// Which dK/dV kernel runs on block lists: the one with 32 keys per wave (two waves per SIMD), or, when the environment
+// asks for it (measurement of that variant), the one with 64 keys per wave (one wave per SIMD).
+hipError_t launch_dkdv_variant(fba::BwdParams& p, hipStream_t stream) {
+  const char* keys = getenv("FBA_DKDV_KEYS_PER_WAVE");
+  if (!p.tiled && keys && atoi(keys) == 64) return fba::launch_bwd_dkdv64(p, stream);
+  return fba::launch_bwd_dkdv(p, stream);
+}
+
 int hip_fail(hipError_t e, const char* what) { return fail(FBA_ERR_HIP, "%s: %s", what, hipGetErrorString(e)); }
+
+// Optional workspace for tail splitting: null (nothing is split), or 16-byte aligned with a non-negative size.
+int check_split_ws(const void* ws, int64_t bytes) {
+  if (ws == nullptr) return FBA_OK;
+  if (!aligned16(ws)) return fail(FBA_ERR_INVALID, "split_ws is not 16-byte aligned");
+  if (bytes < 0) return fail(FBA_ERR_INVALID, "split_ws_bytes must not be negative");
+  return FBA_OK;
+}
 
 }  // namespace
 
@@ -63,6 +79,8 @@ extern "C" {
 int32_t fba_version(void) { return 1000; }
 
 const char* fba_last_error(void) { return g_err; }
+
+int64_t fba_split_workspace_bytes(void) { return fba::kSplitWsBytes; }
 
 int32_t fba_mask_compact(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32_t nK, int32_t* q_cnt, int32_t* q_idx,
                          int32_t* k_cnt, int32_t* k_idx, void* hip_stream) {
@@ -91,12 +109,13 @@ int check_lists(const Shape& s, bool tiled, const char* what) {
 
 int fwd_impl(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* q_cnt, const int32_t* q_idx,
              int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block,
-             int32_t k_block, void* hip_stream, bool tiled) {
+             int32_t k_block, void* split_ws, int64_t split_ws_bytes, void* hip_stream, bool tiled) {
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"o", o}})) return rc;
   if (!lse || !q_cnt || !q_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
   if (int rc = check_lists(s, tiled, "forward")) return rc;
+  if (int rc = check_split_ws(split_ws, split_ws_bytes)) return rc;
   fba::FwdParams p{};
   p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.o = (__bf16*)o; p.lse = lse;
   p.q_cnt = q_cnt; p.q_idx = q_idx; p.mask_bh = mask_bh;
@@ -104,6 +123,7 @@ int fwd_impl(const void* q, const void* k, const void* v, void* o, float* lse, c
   p.q_block = q_block; p.k_block = k_block;
   p.scale_log2e = 1.4426950408889634f / 11.313708498984761f;
   p.tiled = tiled ? 1 : 0;
+  p.split.ws = (float*)split_ws; p.split_ws_bytes = split_ws_bytes;
   {
     const char* rows = getenv("FBA_FWD_TILE_ROWS");
     p.variant = rows && atoi(rows) == 384 ? 0 : 1;  // 128-row work-groups unless asked otherwise
@@ -118,14 +138,15 @@ extern "C" {
 
 int32_t fba_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* q_cnt,
                 const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
-                int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
-  return fwd_impl(q, k, v, o, lse, q_cnt, q_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream, false);
+                int32_t head_dim, int32_t q_block, int32_t k_block, void* split_ws, int64_t split_ws_bytes, void* hip_stream) {
+  return fwd_impl(q, k, v, o, lse, q_cnt, q_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, split_ws, split_ws_bytes,
+                  hip_stream, false);
 }
 
 int32_t fba_fwd_tiled(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* qt_cnt,
                       const int32_t* qt_ent, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
                       int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
-  return fwd_impl(q, k, v, o, lse, qt_cnt, qt_ent, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream, true);
+  return fwd_impl(q, k, v, o, lse, qt_cnt, qt_ent, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, nullptr, 0, hip_stream, true);
 }
 
 int32_t fba_block_mean(const void* x, float* out, int64_t n_seq, int32_t S, int32_t block, int32_t head_dim, void* hip_stream) {
@@ -223,36 +244,41 @@ static int dq_impl(const void* q, const void* k, const void* v, const void* d_o,
 
 static int dkdv_impl(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,
                      const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
-                     int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream, bool tiled) {
+                     int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* split_ws, int64_t split_ws_bytes,
+                     void* hip_stream, bool tiled) {
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"d_o", d_o}, {"dk", dk}, {"dv", dv}})) return rc;
   if (!stats || !k_cnt || !k_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
   if (int rc = check_lists(s, tiled, "dkdv")) return rc;
+  if (int rc = check_split_ws(split_ws, split_ws_bytes)) return rc;
   if ((int64_t)B * Hq * Sq >= (1LL << 30)) return fail(FBA_ERR_INVALID, "B*Hq*Sq must be below 2^30");
   fba::BwdParams p{};
   fill_bwd(p, s);
   p.tiled = tiled ? 1 : 0;
   p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.d_o = (const __bf16*)d_o;
   p.stats = stats; p.dk = (__bf16*)dk; p.dv = (__bf16*)dv; p.k_cnt = k_cnt; p.k_idx = k_idx;
-  hipError_t e = fba::launch_bwd_dkdv(p, (hipStream_t)hip_stream);
+  p.split.ws = (float*)split_ws; p.split_ws_bytes = split_ws_bytes;
+  hipError_t e = launch_dkdv_variant(p, (hipStream_t)hip_stream);
   return e == hipSuccess ? FBA_OK : hip_fail(e, "dkdv launch");
 }
 
 static int bwd_impl(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                     float* stats, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
                     const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
-                    int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream, bool tiled) {
+                    int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* split_ws, int64_t split_ws_bytes,
+                    void* hip_stream, bool tiled) {
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_lists(s, tiled, "backward")) return rc;
+  if (int rc = check_split_ws(split_ws, split_ws_bytes)) return rc;
   // everything is validated before the first launch, so that a rejected call leaves nothing on the stream
   if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"o", o}, {"d_o", d_o}, {"dq", dq}, {"dk", dk}, {"dv", dv}})) return rc;
   if (!lse || !stats || !q_cnt || !q_idx || !k_cnt || !k_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
   if ((int64_t)B * Hq * Sq >= (1LL << 30)) return fail(FBA_ERR_INVALID, "B*Hq*Sq must be below 2^30");
   if (int rc = fba_bwd_stats(o, d_o, lse, stats, (int64_t)B * Hq * Sq, head_dim, hip_stream)) return rc;
   if (int rc = dkdv_impl(q, k, v, d_o, stats, dk, dv, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block,
-                         hip_stream, tiled))
+                         split_ws, split_ws_bytes, hip_stream, tiled))
     return rc;
   return dq_impl(q, k, v, d_o, stats, dq, q_cnt, q_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream, tiled);
 }
@@ -265,16 +291,19 @@ int32_t fba_bwd_dq(const void* q, const void* k, const void* v, const void* d_o,
 
 int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,
                      const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
-                     int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
-  return dkdv_impl(q, k, v, d_o, stats, dk, dv, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream, false);
+                     int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* split_ws, int64_t split_ws_bytes,
+                     void* hip_stream) {
+  return dkdv_impl(q, k, v, d_o, stats, dk, dv, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, split_ws,
+                   split_ws_bytes, hip_stream, false);
 }
 
 int32_t fba_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                 float* stats, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
                 const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
-                int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+                int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* split_ws, int64_t split_ws_bytes,
+                void* hip_stream) {
   return bwd_impl(q, k, v, o, d_o, lse, stats, dq, dk, dv, q_cnt, q_idx, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim,
-                  q_block, k_block, hip_stream, false);
+                  q_block, k_block, split_ws, split_ws_bytes, hip_stream, false);
 }
 
 int32_t fba_probe_mfma(const float* src, float* sink, int32_t work_groups, int32_t iters, void* hip_stream) {
@@ -311,10 +340,12 @@ static int check_handover(const Shape& s, const void* ds_ws, int64_t ds_ws_bytes
 int32_t fba_bwd_dkdv_handover(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,
                               void* ds_ws, int64_t ds_ws_bytes, const int32_t* k_cnt, const int32_t* k_idx, const int32_t* pair_base,
                               int64_t n_pairs, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
-                              int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+                              int32_t head_dim, int32_t q_block, int32_t k_block, void* split_ws, int64_t split_ws_bytes,
+                              void* hip_stream) {
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_handover(s, ds_ws, ds_ws_bytes, pair_base, n_pairs, "dkdv")) return rc;
+  if (int rc = check_split_ws(split_ws, split_ws_bytes)) return rc;
   if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"d_o", d_o}, {"dk", dk}, {"dv", dv}})) return rc;
   if (!stats || !k_cnt || !k_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
   if ((int64_t)B * Hq * Sq >= (1LL << 30)) return fail(FBA_ERR_INVALID, "B*Hq*Sq must be below 2^30");
@@ -323,22 +354,26 @@ int32_t fba_bwd_dkdv_handover(const void* q, const void* k, const void* v, const
   p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.d_o = (const __bf16*)d_o;
   p.stats = stats; p.dk = (__bf16*)dk; p.dv = (__bf16*)dv; p.k_cnt = k_cnt; p.k_idx = k_idx;
   p.ds_ws = (__bf16*)ds_ws; p.pair_base = pair_base;
-  hipError_t e = fba::launch_bwd_dkdv(p, (hipStream_t)hip_stream);
+  p.split.ws = (float*)split_ws; p.split_ws_bytes = split_ws_bytes;
+  hipError_t e = launch_dkdv_variant(p, (hipStream_t)hip_stream);
   return e == hipSuccess ? FBA_OK : hip_fail(e, "dkdv (hand-over) launch");
 }
 
 int32_t fba_bwd_dq_from_ds(const void* k, const void* ds_ws, int64_t ds_ws_bytes, void* dq, const int32_t* q_cnt, const int32_t* q_idx,
                            const int32_t* q_slot, const int32_t* pair_base, int64_t n_pairs, int64_t mask_bh, int32_t B, int32_t Hq,
-                           int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+                           int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* split_ws,
+                           int64_t split_ws_bytes, void* hip_stream) {
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_handover(s, ds_ws, ds_ws_bytes, pair_base, n_pairs, "dq")) return rc;
+  if (int rc = check_split_ws(split_ws, split_ws_bytes)) return rc;
   if (int rc = check_ptrs({{"k", k}, {"dq", dq}})) return rc;
   if (!q_cnt || !q_idx || !q_slot) return fail(FBA_ERR_INVALID, "null pointer argument");
   fba::BwdParams p{};
   fill_bwd(p, s);
   p.k = (const __bf16*)k; p.dq = (__bf16*)dq; p.q_cnt = q_cnt; p.q_idx = q_idx;
   p.ds_ws = (__bf16*)const_cast<void*>(ds_ws); p.pair_base = pair_base; p.q_slot = q_slot;
+  p.split.ws = (float*)split_ws; p.split_ws_bytes = split_ws_bytes;
   hipError_t e = fba::launch_bwd_dq_from_ds(p, (hipStream_t)hip_stream);
   return e == hipSuccess ? FBA_OK : hip_fail(e, "dq (from dS) launch");
 }
@@ -347,20 +382,21 @@ int32_t fba_bwd_handover(const void* q, const void* k, const void* v, const void
                          void* ds_ws, int64_t ds_ws_bytes, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
                          const int32_t* k_cnt, const int32_t* k_idx, const int32_t* pair_base, const int32_t* q_slot, int64_t n_pairs,
                          int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim,
-                         int32_t q_block, int32_t k_block, void* hip_stream) {
+                         int32_t q_block, int32_t k_block, void* split_ws, int64_t split_ws_bytes, void* hip_stream) {
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
   // everything is validated before the first launch, so that a rejected call leaves nothing on the stream
   if (int rc = check_handover(s, ds_ws, ds_ws_bytes, pair_base, n_pairs, "backward")) return rc;
+  if (int rc = check_split_ws(split_ws, split_ws_bytes)) return rc;
   if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"o", o}, {"d_o", d_o}, {"dq", dq}, {"dk", dk}, {"dv", dv}})) return rc;
   if (!lse || !stats || !q_cnt || !q_idx || !k_cnt || !k_idx || !q_slot) return fail(FBA_ERR_INVALID, "null pointer argument");
   if ((int64_t)B * Hq * Sq >= (1LL << 30)) return fail(FBA_ERR_INVALID, "B*Hq*Sq must be below 2^30");
   if (int rc = fba_bwd_stats(o, d_o, lse, stats, (int64_t)B * Hq * Sq, head_dim, hip_stream)) return rc;
   if (int rc = fba_bwd_dkdv_handover(q, k, v, d_o, stats, dk, dv, ds_ws, ds_ws_bytes, k_cnt, k_idx, pair_base, n_pairs, mask_bh, B, Hq,
-                                     Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream))
+                                     Hkv, Sq, Skv, head_dim, q_block, k_block, split_ws, split_ws_bytes, hip_stream))
     return rc;
   return fba_bwd_dq_from_ds(k, ds_ws, ds_ws_bytes, dq, q_cnt, q_idx, q_slot, pair_base, n_pairs, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim,
-                            q_block, k_block, hip_stream);
+                            q_block, k_block, split_ws, split_ws_bytes, hip_stream);
 }
 
 int32_t fba_tile_slots(const int32_t* kt_cnt, const int32_t* kt_ent, int64_t mask_bh, int32_t n_qt, int32_t n_kt, int32_t* pair_base,
@@ -453,7 +489,7 @@ int32_t fba_bwd_noalloc(const void* q, const void* k, const void* v, const void*
   float* stats = nullptr;
   if (int rc = scratch_address(&stats)) return rc;
   return bwd_impl(q, k, v, o, d_o, lse, stats, dq, dk, dv, q_cnt, q_idx, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim,
-                  q_block, k_block, hip_stream, false);
+                  q_block, k_block, nullptr, 0, hip_stream, false);
 }
 
 int32_t fba_bwd_tiled(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
@@ -461,7 +497,7 @@ int32_t fba_bwd_tiled(const void* q, const void* k, const void* v, const void* o
                       const int32_t* kt_cnt, const int32_t* kt_ent, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
                       int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
   return bwd_impl(q, k, v, o, d_o, lse, stats, dq, dk, dv, qt_cnt, qt_ent, kt_cnt, kt_ent, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim,
-                  q_block, k_block, hip_stream, true);
+                  q_block, k_block, nullptr, 0, hip_stream, true);
 }
 
 }  // extern "C"

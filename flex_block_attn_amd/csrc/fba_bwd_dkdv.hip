@@ -54,8 +54,17 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kg = wave & 3, par = wave >> 2;
-  const int item = xcd_remap(blockIdx.x, p.items_per_xcd);
-  if (item >= p.num_items) return;
+  // whole items first (dealt to the XCDs in contiguous spans), then the parts of the split items
+  int item, part = 0, parts = 1;
+  if ((int)blockIdx.x < p.split.main_wgs) {
+    item = xcd_remap(blockIdx.x, p.items_per_xcd);
+    if (item >= p.split.first) return;
+  } else {
+    const int s = blockIdx.x - p.split.main_wgs;
+    item = p.split.first + s / p.split.parts;
+    part = s - (item - p.split.first) * p.split.parts;
+    parts = p.split.parts;
+  }
   const int tiles_per_head = p.Skv / TK;
   const int bhk = item / tiles_per_head;
   const int kt = item - bhk * tiles_per_head;
@@ -71,9 +80,25 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     return (p.mask_bh == 1 ? 0 : bh) * (kTiled ? tiles_per_head : p.nK) + (kTiled ? kt : kblk);
   };
   const ConstIdx k_cnt = const_idx(p.k_cnt);
-  int nslabs = 0;
-  for (int g = 0; g < group; ++g) nslabs += k_cnt[list_row(g)];
-  nslabs *= nsub;
+  int slabs_all = 0;
+  for (int g = 0; g < group; ++g) slabs_all += k_cnt[list_row(g)];
+  slabs_all *= nsub;
+  // this work-group's range of listed slabs: all of them, or part `part` of `parts` (boundaries on multiples of four slabs;
+  // block lists only)
+  const int s_begin = parts == 1 ? 0 : 4 * (int)(((int64_t)(slabs_all / 4) * part) / parts);
+  const int nslabs = (parts == 1 ? slabs_all : 4 * (int)(((int64_t)(slabs_all / 4) * (part + 1)) / parts)) - s_begin;
+  // (query head of the group, list entry, slab inside the query block) of slab s_begin
+  int g_begin = 0, e_begin = 0, sub_begin = 0;
+  if (parts > 1) {
+    int s = s_begin;
+    for (; g_begin < group - 1; ++g_begin) {
+      const int n = k_cnt[list_row(g_begin)] * nsub;
+      if (s < n) break;
+      s -= n;
+    }
+    e_begin = s / nsub;
+    sub_begin = s - e_begin * nsub;
+  }
 
   RowMajorOffsets rm;
   rm.init(lane);
@@ -142,7 +167,18 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
       advance();
       issue_copy(2 * pair_slot + par, par ? r1 : r0);
     };
-    next_block();
+    if (parts == 1) {
+      next_block();
+    } else {  // start in the middle of the lists
+      g_cur = g_begin;
+      const int64_t lr = list_row(g_cur);
+      cnt_cur = k_cnt[lr];
+      idx_cur = const_idx(p.k_idx + lr * row_len);
+      head_row0 = ((int64_t)b * p.Hq + hkv * group + g_cur) * p.Sq;
+      e_cur = e_begin;
+      row_next = head_row0 + (int64_t)idx_cur[e_cur] * p.q_block + sub_begin * kSlab;
+      rem = nsub - sub_begin;
+    }
     request_pair(0);
     request_pair(1);
 
@@ -204,7 +240,18 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
       }
     };
     if constexpr (kHandOver && !kTiled) {
-      ho_next_entry();
+      if (parts == 1) {
+        ho_next_entry();
+      } else {
+        h_g = g_begin;
+        const int64_t lr = list_row(h_g);
+        h_cnt = k_cnt[lr];
+        const ConstIdx pb = const_idx(p.pair_base);
+        const int64_t bh = (int64_t)b * p.Hq + hkv * group + h_g;
+        h_slot0 = pb[lr] + (p.mask_bh == 1 ? bh * pb[p.nK] : 0);
+        h_e = e_begin;
+        h_s = sub_begin;
+      }
       ho_advance(par);
     }
     wait_vmem<0>();
@@ -330,6 +377,19 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
       }
   }
 
+  if (parts > 1) {
+    // part of a split item: unscaled fp32 partial sums go to the workspace, dV tile (parity 0), then dK tile (parity 1)
+    float* prow = p.split.ws + ((int64_t)(item - p.split.first) * parts + part) * (2 * TK * kHeadDim) + par * (TK * kHeadDim) +
+                  (kg * 32 + l32) * kHeadDim;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x16& a = par ? acc_k[mb] : acc_v[mb];
+        *reinterpret_cast<f32x4*>(prow + 32 * mb + 8 * g + 4 * h) = (f32x4){a[4 * g + 0], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
+      }
+    return;
+  }
   // parity 0 writes dV, parity 1 writes dK (both zero when no query block selects this key tile)
   __bf16* orow = (par ? p.dk : p.dv) + (krow0 + kg * 32 + l32) * kHeadDim;
   const float oscale = par ? p.scale : 1.f;
@@ -345,13 +405,23 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
 
 hipError_t launch_bwd_dkdv(BwdParams p, hipStream_t stream) {
   p.num_items = p.B * p.Hkv * (p.Skv / 128);
-  p.items_per_xcd = (p.num_items + kNumXcd - 1) / kNumXcd;
+  // tail splitting on block lists (one work-group per compute unit); a part stores two 128 x 128 fp32 tiles
+  p.split = plan_split(p.num_items, 1, 2 * 128 * kHeadDim * 4, p.tiled ? nullptr : p.split.ws, p.split_ws_bytes);
+  p.items_per_xcd = (p.split.first + kNumXcd - 1) / kNumXcd;
+  p.split.main_wgs = p.items_per_xcd * kNumXcd;
+  const int split_items = p.num_items - p.split.first;
   const bool hand_over = p.ds_ws != nullptr;
   void (*fn)(const BwdParams) = p.tiled ? (hand_over ? &dkdv_kernel<true, true> : &dkdv_kernel<true, false>)
                                         : (hand_over ? &dkdv_kernel<false, true> : &dkdv_kernel<false, false>);
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(fn, dim3(p.items_per_xcd * kNumXcd), dim3(512), kSmemBytes, stream, p);
+  hipLaunchKernelGGL(fn, dim3(p.split.main_wgs + split_items * p.split.parts), dim3(512), kSmemBytes, stream, p);
+  if (split_items > 0) {
+    const int64_t row0 = (int64_t)p.split.first * 128;
+    e = launch_partial_sum(p.split.ws, p.split.parts, 2 * 128 * kHeadDim, p.dv, row0, split_items, 1.f, stream);
+    if (e != hipSuccess) return e;
+    return launch_partial_sum(p.split.ws + 128 * kHeadDim, p.split.parts, 2 * 128 * kHeadDim, p.dk, row0, split_items, p.scale, stream);
+  }
   return hipGetLastError();
 }
 

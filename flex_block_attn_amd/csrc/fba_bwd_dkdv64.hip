@@ -1,0 +1,540 @@
+// Backward, dK and dV, 64 keys per wave: gfx950, head_dim 128, bf16 in / fp32 accumulate / bf16 out, no atomics.
+//
+// Same mathematics, lists, hand-over layout and tail splitting as dkdv_kernel (fba_bwd_dkdv.hip); what differs is the shape
+// of a wave's work.  Work-group = 128 key rows, four waves, one per SIMD.  Wave w works on keys 64 (w % 2) .. +63 (two
+// 32-key groups) and on every second 32-query slab of the list (w / 2 = parity of the slab).  Every Q / dO operand fetched
+// from LDS, row-major or transposed, then feeds two matrix instructions, one per key group, and the K rows of the wave
+// stay in registers for the whole list: 40 KiB of LDS reads per 64 matrix instructions instead of 96 KiB.  The price is
+// one wave per SIMD: dK and dV accumulators alone are 256 registers per lane (kept in accumulation registers), and
+// nothing but the wave's own instruction order overlaps softmax arithmetic with matrix work.
+// LDS: ring of six (Q slab | dO slab | lse2 | -delta) buffers, three per slab parity, then the V tile (32 KiB).
+#include <type_traits>
+
+#include "fba_common.h"
+#include "fba_kernels.h"
+
+namespace fba {
+
+namespace {
+
+constexpr int kSlab = 32;
+constexpr int kSlabBytes = kSlab * kRowBytes;       // 8 KiB
+constexpr int kStatBytes = 2 * kSlab * 4;           // lse2[32] | -delta[32]
+constexpr int kStageBytes = 2 * kSlabBytes + kStatBytes;
+constexpr int kRing = 6;                            // three buffers per slab parity
+constexpr int kTileBytes = 128 * kRowBytes;         // K or V tile, 32 KiB
+constexpr int kRingBase = 0;                        // the ring first: its offsets fit the 16-bit field of an LDS fetch
+constexpr int kTileBase = kRing * kStageBytes;      // V tile
+constexpr int kSmemBytes = kTileBase + kTileBytes;   // ring + V tile (130 KiB); the final exchange re-uses the first 128 KiB
+
+template <int N>
+using IC = std::integral_constant<int, N>;
+
+// acc += a b with the accumulator held in accumulation registers.  dK and dV of 64 keys are 256 registers per lane, all
+// the accumulation registers a wave has; S and dP, which the softmax arithmetic reads, must therefore live in ordinary
+// registers, and the compiler does not mix the two forms of the instruction on its own.  Written as inline asm, so the
+// compiler does not know that it is a matrix instruction and inserts none of the wait states one needs; that is safe
+// here because (a) its A and B operands come from LDS fetches and from conversion instructions, never straight from
+// another matrix instruction, (b) two of these on one accumulator are always at least eight matrix instructions apart,
+// and (c) the accumulators are read only after drain_matrix_pipe() below.
+FBA_DEVICE void mfma32_acc(f32x16& acc, bf16x8 a, bf16x8 b) {
+  asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+// More idle cycles than any matrix instruction needs to retire its result.
+FBA_DEVICE void drain_matrix_pipe() { asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15" ::: "memory"); }
+
+}  // namespace
+
+// Block lists only (q_block and k_block multiples of 128; list entries are query blocks, expanded to q_block/32 slabs).
+// kHandOver: every wave also stores the bf16 dS it forms to p.ds_ws (layout: fba_common.h), so that dQ = dS K can be
+// formed later without recomputing S and dP.
+template <bool kHandOver>
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_per_eu(1, 1))) void dkdv64_kernel(const BwdParams p) {
+  constexpr bool kTiled = false;
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  constexpr int TK = 128;
+
+  const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int kg = wave & 1, par = wave >> 1;  // 64-key group, slab parity
+  // whole items first (dealt to the XCDs in contiguous spans), then the parts of the split items
+  int item, part = 0, parts = 1;
+  if ((int)blockIdx.x < p.split.main_wgs) {
+    item = xcd_remap(blockIdx.x, p.items_per_xcd);
+    if (item >= p.split.first) return;
+  } else {
+    const int s = blockIdx.x - p.split.main_wgs;
+    item = p.split.first + s / p.split.parts;
+    part = s - (item - p.split.first) * p.split.parts;
+    parts = p.split.parts;
+  }
+  const int tiles_per_head = p.Skv / TK;
+  const int bhk = item / tiles_per_head;
+  const int kt = item - bhk * tiles_per_head;
+  const int b = bhk / p.Hkv, hkv = bhk - b * p.Hkv;
+  const int group = p.Hq / p.Hkv;
+  const int kblk = (kt * TK) / p.k_block;
+  const int64_t krow0 = (int64_t)bhk * p.Skv + (int64_t)kt * TK;
+
+  const int nsub = kTiled ? 1 : p.q_block / kSlab;
+  const int row_len = kTiled ? p.Sq / kSlab : p.nQ;  // entries per list row
+  auto list_row = [&](int g) -> int64_t {
+    const int64_t bh = (int64_t)b * p.Hq + hkv * group + g;
+    return (p.mask_bh == 1 ? 0 : bh) * (kTiled ? tiles_per_head : p.nK) + (kTiled ? kt : kblk);
+  };
+  const ConstIdx k_cnt = const_idx(p.k_cnt);
+  int slabs_all = 0;
+  for (int g = 0; g < group; ++g) slabs_all += k_cnt[list_row(g)];
+  slabs_all *= nsub;
+  // this work-group's range of listed slabs: all of them, or part `part` of `parts` (boundaries on multiples of four slabs;
+  // block lists only)
+  const int s_begin = parts == 1 ? 0 : 4 * (int)(((int64_t)(slabs_all / 4) * part) / parts);
+  const int nslabs = (parts == 1 ? slabs_all : 4 * (int)(((int64_t)(slabs_all / 4) * (part + 1)) / parts)) - s_begin;
+  // (query head of the group, list entry, slab inside the query block) of slab s_begin
+  int g_begin = 0, e_begin = 0, sub_begin = 0;
+  if (parts > 1) {
+    int s = s_begin;
+    for (; g_begin < group - 1; ++g_begin) {
+      const int n = k_cnt[list_row(g_begin)] * nsub;
+      if (s < n) break;
+      s -= n;
+    }
+    e_begin = s / nsub;
+    sub_begin = s - e_begin * nsub;
+  }
+
+  RowMajorOffsets rm;
+  rm.init(lane);
+  TransposedOffsets tr;
+  tr.init(lane);
+  // the two waves of a parity bring in a slab together, 16 rows (four wave-level copies) each
+  uint32_t dma_off[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) {
+    const int row = 16 * kg + 4 * g + (lane >> 4);
+    dma_off[g] = (uint32_t)(row * kRowBytes + (((lane & 15) ^ swz(row)) << 4));
+  }
+  const uint32_t dma_dst = (uint32_t)(16 * kg * kRowBytes);
+  auto copy_slab = [&](uint32_t slab_lds, const char* src) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g) dma16(slab_lds + dma_dst + g * 4 * kRowBytes, src, dma_off[g]);
+  };
+  const uint32_t lds0 = lds_addr(smem);
+  const uint32_t ring_dst = lds0 + kRingBase;
+  const int64_t rows_total = (int64_t)p.B * p.Hq * p.Sq;
+  // statistics copy: lanes 0..31 fetch lse2[row0 + l], lanes 32..63 fetch -delta[row0 + l - 32]
+  const uint32_t stat_off = (uint32_t)((lane >> 5) * rows_total * 4 + (lane & 31) * 4);
+  const float c = p.scale_log2e;
+
+  f32x16 acc_k[2][4], acc_v[2][4];  // [32-key group][32 head-dim columns]
+#pragma unroll
+  for (int grp = 0; grp < 2; ++grp)
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { acc_k[grp][mb][r] = 0.f; acc_v[grp][mb][r] = 0.f; }
+
+  if (nslabs > 0) {
+    // V tile into LDS: wave w brings in rows 32 w .. 32 w + 31 (two slabs' worth of copies)
+    {
+      const char* src = reinterpret_cast<const char*>(p.v) + (krow0 + 32 * wave) * kRowBytes;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const uint32_t dst = lds0 + kTileBase + wave * kSlabBytes + j * 16 * kRowBytes;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int row = 4 * g + (lane >> 4);  // row inside the 16-row half; swz depends on row % 16 only
+          dma16(dst + g * 4 * kRowBytes, src + j * 16 * kRowBytes, (uint32_t)(row * kRowBytes + (((lane & 15) ^ swz(row)) << 4)));
+        }
+      }
+    }
+    // K rows of the wave's two key groups as B operands, in registers for the whole list: lane holds key l32 of the group,
+    // d = 16 ks + 8 h .. +7
+    bf16x8 kreg[2][8];
+    {
+      const __bf16* kp = p.k + (krow0 + 64 * kg + l32) * kHeadDim + 8 * h;
+#pragma unroll
+      for (int grp = 0; grp < 2; ++grp)
+#pragma unroll
+        for (int ks = 0; ks < 8; ++ks) kreg[grp][ks] = *reinterpret_cast<const bf16x8*>(kp + grp * 32 * kHeadDim + 16 * ks);
+    }
+    // Cursor over (query head of the group, list entry, slab): first query row of the next slab to request.
+    const char* qbase = reinterpret_cast<const char*>(p.q);
+    const char* dobase = reinterpret_cast<const char*>(p.d_o);
+    const char* stbase = reinterpret_cast<const char*>(p.stats);
+    int g_cur = -1, e_cur = -1, cnt_cur = 0, rem = 1;
+    bool more = true;  // false once every listed slab has been requested; row_next then stays on the last one
+    ConstIdx idx_cur = nullptr;
+    int64_t row_next = 0, head_row0 = 0;
+    auto next_block = [&]() {  // position row_next on the first row of the next listed query block, if any
+      ++e_cur;
+      while (e_cur >= cnt_cur) {
+        if (++g_cur >= group) { more = false; return; }
+        const int64_t lr = list_row(g_cur);
+        cnt_cur = k_cnt[lr];
+        idx_cur = const_idx(p.k_idx + lr * row_len);
+        head_row0 = ((int64_t)b * p.Hq + hkv * group + g_cur) * p.Sq;
+        e_cur = 0;
+      }
+      row_next = head_row0 + (kTiled ? (int64_t)(idx_cur[e_cur] >> 8) * kSlab : (int64_t)idx_cur[e_cur] * p.q_block);
+      rem = nsub;
+    };
+    auto advance = [&]() {
+      if (!more) return;
+      if (--rem == 0) next_block(); else row_next += kSlab;
+    };
+    // Nine copies per wave request one slab (Q rows, dO rows, statistics), by the two waves of the slab's parity.  Every
+    // step issues them, so that the count of copies in flight is the same at every wait; once the lists are exhausted
+    // the last slab is simply requested again, into a buffer nobody reads any more.
+    auto issue_copy = [&](int ring, int64_t row) {
+      const uint32_t dst = ring_dst + ring * kStageBytes;
+      copy_slab(dst, qbase + row * kRowBytes);
+      copy_slab(dst + kSlabBytes, dobase + row * kRowBytes);
+      dma4(dst + 2 * kSlabBytes, stbase + row * 4, stat_off);  // both waves copy the same 256 bytes
+    };
+    // the same request one copy at a time (i = 0..8), for spreading over a phase of matrix instructions
+    auto issue_copy_part = [&](int i, uint32_t dst, int64_t row) {
+      if (i < 4) dma16(dst + dma_dst + i * 4 * kRowBytes, qbase + row * kRowBytes, dma_off[i]);
+      else if (i < 8) dma16(dst + kSlabBytes + dma_dst + (i - 4) * 4 * kRowBytes, dobase + row * kRowBytes, dma_off[i - 4]);
+      else dma4(dst + 2 * kSlabBytes, stbase + row * 4, stat_off);
+    };
+    // Slabs are numbered in list order; slabs 2i and 2i+1 form pair i, the first for the waves of parity 0, the second for
+    // those of parity 1.  A parity keeps three buffers: ring buffer 3 * par + (i % 3) holds its slab of pair i.
+    auto request_pair = [&](int buf) {
+      const int64_t r0 = row_next;
+      advance();
+      const int64_t r1 = row_next;
+      advance();
+      issue_copy(3 * par + buf, par ? r1 : r0);
+    };
+    if (parts == 1) {
+      next_block();
+    } else {  // start in the middle of the lists
+      g_cur = g_begin;
+      const int64_t lr = list_row(g_cur);
+      cnt_cur = k_cnt[lr];
+      idx_cur = const_idx(p.k_idx + lr * row_len);
+      head_row0 = ((int64_t)b * p.Hq + hkv * group + g_cur) * p.Sq;
+      e_cur = e_begin;
+      row_next = head_row0 + (int64_t)idx_cur[e_cur] * p.q_block + sub_begin * kSlab;
+      rem = nsub - sub_begin;
+    }
+    request_pair(0);
+    request_pair(1);
+
+    // dS hand-over: (query head of the group, list entry, slab inside the query block) of the slab whose dS this wave forms
+    // next, and the pair number of entry 0 of that head's list row
+    int h_g = -1, h_e = -1, h_s = 0, h_cnt = 0;
+    int64_t h_slot0 = 0;
+    const int64_t pair_bytes = (int64_t)p.q_block * p.k_block * 2;
+    const int nsub_k = p.k_block / kSlab;
+    const int t_key = 4 * ((kt * TK - kblk * p.k_block) / TK) + 2 * kg;  // this wave's first 32-key slab inside the key block
+    const int ho_off0 = ds_unit_store_off(0, lane), ho_off1 = ds_unit_store_off(1, lane);
+    auto ho_next_entry = [&]() {
+      ++h_e;
+      while (h_e >= h_cnt) {
+        if (++h_g >= group) return;
+        const int64_t lr = list_row(h_g);
+        h_cnt = k_cnt[lr];
+        const ConstIdx pb = const_idx(p.pair_base);
+        const int64_t bh = (int64_t)b * p.Hq + hkv * group + h_g;
+        h_slot0 = pb[lr] + (p.mask_bh == 1 ? bh * pb[p.nK] : 0);
+        h_e = 0;
+      }
+    };
+    auto ho_advance = [&](int n) {
+      h_s += n;
+      if (h_s >= nsub) {  // nsub >= 4 > n
+        h_s -= nsub;
+        ho_next_entry();
+      }
+    };
+    if constexpr (kHandOver) {
+      if (parts == 1) {
+        ho_next_entry();
+      } else {
+        h_g = g_begin;
+        const int64_t lr = list_row(h_g);
+        h_cnt = k_cnt[lr];
+        const ConstIdx pb = const_idx(p.pair_base);
+        const int64_t bh = (int64_t)b * p.Hq + hkv * group + h_g;
+        h_slot0 = pb[lr] + (p.mask_bh == 1 ? bh * pb[p.nK] : 0);
+        h_e = e_begin;
+        h_s = sub_begin;
+      }
+      ho_advance(par);
+    }
+    wait_vmem<0>();
+    __syncthreads();
+
+    // per-lane fetch addresses with the wave's share folded in: slab addresses carry the parity's three buffers, V
+    // addresses the wave's 64 keys; what remains (buffer, Q or dO, key group, row group) is a compile-time displacement
+    const LdsPtr lds = lds_ptr(smem);
+    LdsPtr q_ptr[8], v_ptr[8], t_ptr[4][2];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+      q_ptr[ks] = lds + rm.rd[ks] + par * 3 * kStageBytes;
+      v_ptr[ks] = lds + rm.rd[ks] + kTileBase + kg * 2 * kSlabBytes;
+    }
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb) {
+      t_ptr[mb][0] = lds + tr.rd[mb][0] + par * 3 * kStageBytes;
+      t_ptr[mb][1] = lds + tr.rd[mb][1] + par * 3 * kStageBytes;
+    }
+    const LdsPtr st_ptr = lds + par * 3 * kStageBytes + 2 * kSlabBytes + 16 * h;
+#pragma unroll
+    for (int grp = 0; grp < 2; ++grp)
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) pin(kreg[grp][ks]);
+
+    // Software pipeline over the wave's slabs t = 0, 1, ...: while the vector unit turns S_t, dP_t into P_t, dS_t, the matrix
+    // pipe adds slab t-1 into dV and dK; then it forms S_{t+1}, dP_{t+1}.  One wave per SIMD has nobody else to hide behind,
+    // so the interleaving is written out: one accumulating matrix instruction, then the arithmetic of one accumulator
+    // element of both products, each anchored in place.
+    f32x16 s[2], dp[2];
+    bf16x8 pk[2][2], dsk[2][2];  // P and dS of the previous slab, packed as B operands
+
+    // S, dP of the slab in the buffer at byte offset `so` against this wave's 64 keys: every Q / dO operand feeds both key
+    // groups.  The operands of step ks+1 are requested before the matrix instructions of step ks are issued; the scheduling
+    // fences keep the compiler from moving them back next to their use, where the wave would wait for every fetch.
+    auto scores = [&](int so, bool request, uint32_t req_dst, int64_t req_row, char* ds_unit) {
+      // accumulator element 4g + e of half-wave h is query row 8g + 4h + e of the slab; dP starts from -delta of its row
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 d4 = lds_read_f32x4(st_ptr + so + 4 * kSlab + 32 * g);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          s[0][4 * g + e] = 0.f; s[1][4 * g + e] = 0.f;
+          dp[0][4 * g + e] = d4[e]; dp[1][4 * g + e] = d4[e];
+        }
+      }
+      bf16x8 qf = lds_read_b128(q_ptr[0] + so), dof = lds_read_b128(q_ptr[0] + so + kSlabBytes);
+      bf16x8 vf0 = lds_read_b128(v_ptr[0]), vf1 = lds_read_b128(v_ptr[0] + kSlabBytes);
+#pragma unroll
+      for (int ks = 0; ks < 8; ++ks) {
+        bf16x8 qf_n = qf, dof_n = dof, vf0_n = vf0, vf1_n = vf1;
+        if (ks < 7) {
+          qf_n = lds_read_b128(q_ptr[ks + 1] + so);
+          dof_n = lds_read_b128(q_ptr[ks + 1] + so + kSlabBytes);
+          vf0_n = lds_read_b128(v_ptr[ks + 1]);
+          vf1_n = lds_read_b128(v_ptr[ks + 1] + kSlabBytes);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        s[0] = mfma32(qf, kreg[0][ks], s[0]);
+        s[1] = mfma32(qf, kreg[1][ks], s[1]);
+        // the copies of the slab after next and the dS stores of the slab before are issued one at a time between the
+        // matrix instructions: a wave alone on its SIMD pays for every cycle a memory instruction takes to issue
+        // (copies first, stores last: the wait before the next barrier then lets the four youngest operations, the stores,
+        // stay in flight)
+        if (ks < 4) {
+          if (request) issue_copy_part(2 * ks, req_dst, req_row);
+        }
+        dp[0] = mfma32(dof, vf0, dp[0]);
+        if (ks < 4) {
+          if (request) issue_copy_part(2 * ks + 1, req_dst, req_row);
+        } else if (ks == 4) {
+          if (request) issue_copy_part(8, req_dst, req_row);
+        }
+        dp[1] = mfma32(dof, vf1, dp[1]);
+        if constexpr (kHandOver) {
+          if (ks >= 4 && ds_unit != nullptr)
+            __builtin_nontemporal_store(dsk[(ks >> 1) & 1][ks & 1],
+                                        reinterpret_cast<bf16x8*>(ds_unit + ((ks >> 1) & 1) * 4 * kDsUnitBytes + ((ks & 1) ? ho_off1 : ho_off0)));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        qf = qf_n; dof = dof_n; vf0 = vf0_n; vf1 = vf1_n;
+      }
+    };
+
+    // P_t, dS_t from s, dp (statistics in the buffer at `so`), interleaved with dV += dO^T P, dK += Q^T dS of the previous
+    // slab (buffer at `po`, operands pk / dsk).  Eight groups of four
+    // matrix instructions (one transposed dO operand and one transposed Q operand, each against both key groups) and four
+    // accumulator elements of arithmetic; the operands and statistics of group n+1 are requested before group n starts.
+    auto softmax_and_accumulate = [&](int so, int po) {
+      bf16x2 pw[2][8], dw[2][8];  // new P and dS, packed: [key group][register pair]
+      auto fetch_dv = [&](int n) {
+        const int roff = po + 16 * (n >> 2) * kRowBytes, mb = n & 3;
+        return cat(lds_read_tr(t_ptr[mb][0] + kSlabBytes + roff), lds_read_tr(t_ptr[mb][1] + kSlabBytes + roff));
+      };
+      auto fetch_dk = [&](int n) {
+        const int roff = po + 16 * (n >> 2) * kRowBytes, mb = n & 3;
+        return cat(lds_read_tr(t_ptr[mb][0] + roff), lds_read_tr(t_ptr[mb][1] + roff));
+      };
+      bf16x8 adv = fetch_dv(0), adk = fetch_dk(0);
+      f32x4 l4 = lds_read_f32x4(st_ptr + so);
+#pragma unroll
+      for (int n = 0; n < 8; ++n) {  // n = 4 j + mb for the matrix work, 4 grp + g for the arithmetic
+        bf16x8 adv_n = adv, adk_n = adk;
+        f32x4 l4_n = l4;
+        if (n < 7) {
+          adv_n = fetch_dv(n + 1);
+          adk_n = fetch_dk(n + 1);
+          l4_n = lds_read_f32x4(st_ptr + so + 32 * ((n + 1) & 3));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        const int j = n >> 2, mb = n & 3, grp = n >> 2, g = n & 3;
+        float pv[4], dsv[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (e == 0) mfma32_acc(acc_v[0][mb], adv, pk[0][j]);
+          if (e == 1) mfma32_acc(acc_v[1][mb], adv, pk[1][j]);
+          if (e == 2) mfma32_acc(acc_k[0][mb], adk, dsk[0][j]);
+          if (e == 3) mfma32_acc(acc_k[1][mb], adk, dsk[1][j]);
+          pv[e] = fast_exp2(__builtin_fmaf(s[grp][4 * g + e], c, -l4[e]));
+          dsv[e] = pv[e] * dp[grp][4 * g + e];
+          if (e & 1) {
+            bf16x2 p2 = __builtin_convertvector((f32x2){pv[e - 1], pv[e]}, bf16x2);
+            bf16x2 d2 = __builtin_convertvector((f32x2){dsv[e - 1], dsv[e]}, bf16x2);
+            asm volatile("" : "+v"(p2), "+v"(d2));
+            pw[grp][2 * g + (e >> 1)] = p2;
+            dw[grp][2 * g + (e >> 1)] = d2;
+          } else {
+            asm volatile("" : "+v"(pv[e]), "+v"(dsv[e]));  // keeps this element's arithmetic behind its matrix instruction
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        adv = adv_n; adk = adk_n; l4 = l4_n;
+      }
+#pragma unroll
+      for (int grp = 0; grp < 2; ++grp)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          pk[grp][j] = cat(__builtin_shufflevector(pw[grp][4 * j + 0], pw[grp][4 * j + 1], 0, 1, 2, 3),
+                           __builtin_shufflevector(pw[grp][4 * j + 2], pw[grp][4 * j + 3], 0, 1, 2, 3));
+          dsk[grp][j] = cat(__builtin_shufflevector(dw[grp][4 * j + 0], dw[grp][4 * j + 1], 0, 1, 2, 3),
+                            __builtin_shufflevector(dw[grp][4 * j + 2], dw[grp][4 * j + 3], 0, 1, 2, 3));
+        }
+    };
+
+    const int nlocal = nslabs >> 1;  // slabs of this wave's parity (nslabs is a multiple of four)
+#pragma unroll
+    for (int grp = 0; grp < 2; ++grp)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { pk[grp][j][e] = (__bf16)0.f; dsk[grp][j][e] = (__bf16)0.f; }
+    scores(0, false, 0, 0, nullptr);
+    // Iteration t: slab t lives in buffer t % 3, slab t-1 in (t+2) % 3, slab t+1 in (t+1) % 3.  The first iteration adds
+    // nothing (P = dS = 0 against the finite rows of slab 0); the last one, t = nlocal, only adds slab nlocal-1 (its
+    // arithmetic runs on stale registers and is dropped), so that every wave passes the same barriers.
+    int cur = 0, prev = 0, nxt = kStageBytes;
+    bool stores_in_flight = false;  // did the previous iteration end with four dS stores?
+    for (int t = 0; t <= nlocal; ++t) {
+      softmax_and_accumulate(cur, prev);
+      char* ds_unit = nullptr;  // where dS_t goes (null: nothing to store)
+      if constexpr (kHandOver) {
+        if (t < nlocal)
+          ds_unit = reinterpret_cast<char*>(p.ds_ws) + (h_slot0 + h_e) * pair_bytes +
+                    ((int64_t)((h_s >> 2) * nsub_k + t_key) * 4 + (h_s & 3)) * kDsUnitBytes;
+        ho_advance(2);
+      }
+      // this wave's copies of slab t+1, requested during the previous iteration, must have landed; the four dS stores issued
+      // after them may still be on their way (the counter covers loads and stores alike, in issue order)
+      if (kHandOver && stores_in_flight) wait_vmem<4>(); else wait_vmem<0>();
+      __syncthreads();  // everybody is done with slab t-1 and everybody's copies of slab t+1 have landed
+      const int freed = nxt + kStageBytes == 3 * kStageBytes ? 0 : nxt + kStageBytes;  // buffer of slab t-1 = buffer of slab t+2
+      // slab t+2 replaces slab t-1, if the wave has one; its copies are issued in between the matrix instructions of scores()
+      const int64_t r0 = row_next;
+      advance();
+      const int64_t r1 = row_next;
+      advance();
+      const bool request = t + 2 < nlocal;
+      const uint32_t req_dst = ring_dst + 3 * par * kStageBytes + freed;
+      stores_in_flight = ds_unit != nullptr;
+      if (t + 1 < nlocal) {
+        scores(nxt, request, req_dst, par ? r1 : r0, ds_unit);
+      } else if constexpr (kHandOver) {
+        if (ds_unit != nullptr) {  // the wave's last slab: no scores() follows that could carry its stores
+#pragma unroll
+          for (int grp = 0; grp < 2; ++grp) {
+            __builtin_nontemporal_store(dsk[grp][0], reinterpret_cast<bf16x8*>(ds_unit + grp * 4 * kDsUnitBytes + ho_off0));
+            __builtin_nontemporal_store(dsk[grp][1], reinterpret_cast<bf16x8*>(ds_unit + grp * 4 * kDsUnitBytes + ho_off1));
+          }
+        }
+      }
+      prev = cur;
+      cur = nxt;
+      nxt = freed;
+    }
+    wait_vmem<0>();
+    __syncthreads();  // no copy is writing LDS any more; V and the ring are free
+
+    drain_matrix_pipe();
+    // The two waves of a key group swap halves: parity 1 hands its dV part to parity 0 through the first 64 KiB of LDS,
+    // parity 0 hands its dK part to parity 1 through the next 64 KiB (32 KiB per wave each).
+    f32x4* send = reinterpret_cast<f32x4*>(smem + (par ? 0 : 65536) + kg * 32768) + lane;
+    const f32x4* recv = reinterpret_cast<const f32x4*>(smem + (par ? 65536 : 0) + kg * 32768) + lane;
+#pragma unroll
+    for (int grp = 0; grp < 2; ++grp)
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x16& a = par ? acc_v[grp][mb] : acc_k[grp][mb];
+          send[((grp * 4 + mb) * 4 + g) * 64] = (f32x4){a[4 * g + 0], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
+        }
+    __syncthreads();
+#pragma unroll
+    for (int grp = 0; grp < 2; ++grp)
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x4 r = recv[((grp * 4 + mb) * 4 + g) * 64];
+          f32x16& a = par ? acc_k[grp][mb] : acc_v[grp][mb];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) a[4 * g + e] += r[e];
+        }
+  }
+
+  if (parts > 1) {
+    // part of a split item: unscaled fp32 partial sums go to the workspace, dV tile (parity 0), then dK tile (parity 1)
+    float* prow = p.split.ws + ((int64_t)(item - p.split.first) * parts + part) * (2 * TK * kHeadDim) + par * (TK * kHeadDim) +
+                  (kg * 64 + l32) * kHeadDim;
+#pragma unroll
+    for (int grp = 0; grp < 2; ++grp)
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f32x16& a = par ? acc_k[grp][mb] : acc_v[grp][mb];
+          *reinterpret_cast<f32x4*>(prow + grp * 32 * kHeadDim + 32 * mb + 8 * g + 4 * h) = (f32x4){a[4 * g + 0], a[4 * g + 1], a[4 * g + 2], a[4 * g + 3]};
+        }
+    return;
+  }
+  // parity 0 writes dV, parity 1 writes dK (both zero when no query block selects this key tile)
+  __bf16* orow = (par ? p.dk : p.dv) + (krow0 + kg * 64 + l32) * kHeadDim;
+  const float oscale = par ? p.scale : 1.f;
+#pragma unroll
+  for (int grp = 0; grp < 2; ++grp)
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x16& a = par ? acc_k[grp][mb] : acc_v[grp][mb];
+        *reinterpret_cast<bf16x4*>(orow + grp * 32 * kHeadDim + 32 * mb + 8 * g + 4 * h) =
+            pack4(a[4 * g + 0] * oscale, a[4 * g + 1] * oscale, a[4 * g + 2] * oscale, a[4 * g + 3] * oscale);
+      }
+}
+
+hipError_t launch_bwd_dkdv64(BwdParams p, hipStream_t stream) {
+  p.num_items = p.B * p.Hkv * (p.Skv / 128);
+  // tail splitting (one work-group per compute unit); a part stores two 128 x 128 fp32 tiles
+  p.split = plan_split(p.num_items, 1, 2 * 128 * kHeadDim * 4, p.split.ws, p.split_ws_bytes);
+  p.items_per_xcd = (p.split.first + kNumXcd - 1) / kNumXcd;
+  p.split.main_wgs = p.items_per_xcd * kNumXcd;
+  const int split_items = p.num_items - p.split.first;
+  void (*fn)(const BwdParams) = p.ds_ws != nullptr ? &dkdv64_kernel<true> : &dkdv64_kernel<false>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(fn, dim3(p.split.main_wgs + split_items * p.split.parts), dim3(256), kSmemBytes, stream, p);
+  if (split_items > 0) {
+    const int64_t row0 = (int64_t)p.split.first * 128;
+    e = launch_partial_sum(p.split.ws, p.split.parts, 2 * 128 * kHeadDim, p.dv, row0, split_items, 1.f, stream);
+    if (e != hipSuccess) return e;
+    return launch_partial_sum(p.split.ws + 128 * kHeadDim, p.split.parts, 2 * 128 * kHeadDim, p.dk, row0, split_items, p.scale, stream);
+  }
+  return hipGetLastError();
+}
+
+}  // namespace fba

@@ -44,8 +44,17 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int item = xcd_remap(blockIdx.x, p.items_per_xcd);
-  if (item >= p.num_items) return;
+  // whole items first (dealt to the XCDs in contiguous spans), then the parts of the split items
+  int item, part = 0, parts = 1;
+  if ((int)blockIdx.x < p.split.main_wgs) {
+    item = xcd_remap(blockIdx.x, p.items_per_xcd);
+    if (item >= p.split.first) return;
+  } else {
+    const int s = blockIdx.x - p.split.main_wgs;
+    item = p.split.first + s / p.split.parts;
+    part = s - (item - p.split.first) * p.split.parts;
+    parts = p.split.parts;
+  }
   const int tiles_per_head = p.Sq / TQ;
   const int bh = item / tiles_per_head;
   const int qt = item - bh * tiles_per_head;
@@ -64,7 +73,12 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   // block lists: pair number per list entry; tile lists: pair number per key tile, for this query tile
   const ConstIdx slot = const_idx(p.q_slot + mrow * (kTiled ? n_kt : p.nK));
   const int nsub = p.k_block / kSlab;
-  const int nsteps = cnt * nsub;
+  // this work-group's range of 32-key steps of the list: all of it, or part `part` of `parts` (boundaries on whole rings)
+  const int steps_all = cnt * nsub;
+  const int t_begin = parts == 1 ? 0 : 4 * (int)(((int64_t)(steps_all / 4) * part) / parts);
+  const int t_end = parts == 1 ? steps_all : 4 * (int)(((int64_t)(steps_all / 4) * (part + 1)) / parts);
+  const int nsteps = t_end - t_begin;
+  const int e_begin = t_begin / nsub, sub_begin = t_begin - e_begin * nsub;
   const int64_t pair_bytes = kTiled ? 16 * kDsUnitBytes : (int64_t)p.q_block * p.k_block * 2;
   // dS of this wave's 32 rows: pair base + (tq * nsub + t) * 4 units + wave, t = 32-key slab inside the key block (inside
   // the key tile with tile lists)
@@ -98,11 +112,11 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 
   // sources of the next stage to request, in list order; the following list entry is read one block ahead
   const int64_t block_bytes = (int64_t)p.k_block * kRowBytes;
-  int e_next = 1, rem = nsub;
-  int64_t k_off = cnt > 0 ? key_block(0) * block_bytes : 0;
-  int64_t ds_off_g = cnt > 0 && !kTiled ? slot[0] * pair_bytes : 0;
-  int blk_next = cnt > 1 ? key_block(1) : 0;
-  int slot_next = cnt > 1 && !kTiled ? slot[1] : 0;
+  int e_next = e_begin + 1, rem = nsub - sub_begin;
+  int64_t k_off = nsteps > 0 ? key_block(e_begin) * block_bytes + (int64_t)sub_begin * kSlabBytes : 0;
+  int64_t ds_off_g = nsteps > 0 && !kTiled ? slot[e_begin] * pair_bytes + (int64_t)sub_begin * (4 * kDsUnitBytes) : 0;
+  int blk_next = e_next < cnt ? key_block(e_next) : 0;
+  int slot_next = e_next < cnt && !kTiled ? slot[e_next] : 0;
   // tile lists: predicate bits of the entry being requested and of the next one; pair number of the key tile that the
   // next stage's slab lies in, read one stage ahead
   int bits_req = kTiled && cnt > 0 ? idx[0] & 255 : 0;
@@ -184,6 +198,15 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     }
   }
 
+  if (parts > 1) {  // part of a split item: unscaled fp32 partial sums go to the workspace
+    float* prow = p.split.ws + ((int64_t)(item - p.split.first) * parts + part) * (TQ * kHeadDim) + (wave * 32 + l32) * kHeadDim;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        *reinterpret_cast<f32x4*>(prow + 32 * mb + 8 * g + 4 * h) = (f32x4){acc[mb][4 * g + 0], acc[mb][4 * g + 1], acc[mb][4 * g + 2], acc[mb][4 * g + 3]};
+    return;
+  }
   __bf16* orow = p.dq + (qrow0 + l32) * kHeadDim;
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb)
@@ -222,17 +245,44 @@ hipError_t zero_unit_address(const char** out) {
 
 }  // namespace
 
+// Sums the fp32 partial tiles of the split items in part order: out = scale * sum_p partial_p, as bf16.  One thread per
+// four columns; `rows_per_slot` rows of 128 columns per part, `sections` consecutive outputs per slot (dK/dV: two).
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void partial_sum_kernel(const float* ws, int parts, int64_t slot_floats,
+                                                                                          __bf16* out, int64_t out_row0, float scale) {
+  const int tid = threadIdx.x;
+  const int64_t row = (int64_t)blockIdx.x * 8 + (tid >> 5);  // row among 128 * (split items) rows
+  const int c4 = (tid & 31) * 4;
+  const int64_t it = row >> 7;
+  const int r = (int)(row & 127);
+  const float* src = ws + it * parts * slot_floats + r * kHeadDim + c4;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int q = 0; q < parts; ++q) acc += *reinterpret_cast<const f32x4*>(src + q * slot_floats);
+  *reinterpret_cast<bf16x4*>(out + (out_row0 + row) * kHeadDim + c4) = pack4(acc[0] * scale, acc[1] * scale, acc[2] * scale, acc[3] * scale);
+}
+
+hipError_t launch_partial_sum(const float* ws, int parts, int64_t slot_floats, __bf16* out, int64_t out_row0, int n_items, float scale,
+                              hipStream_t stream) {
+  hipLaunchKernelGGL(partial_sum_kernel, dim3(n_items * 16), dim3(256), 0, stream, ws, parts, slot_floats, out, out_row0, scale);
+  return hipGetLastError();
+}
+
 hipError_t launch_bwd_dq_from_ds(BwdParams p, hipStream_t stream) {
   constexpr int kSmem = kRing * kStageBytes;
   if (p.ds_ws == nullptr) return hipErrorInvalidValue;
   p.num_items = p.B * p.Hq * (p.Sq / 128);
-  p.items_per_xcd = (p.num_items + kNumXcd - 1) / kNumXcd;
+  // tail splitting on block lists (two work-groups per compute unit); a part stores a 128 x 128 fp32 tile
+  p.split = plan_split(p.num_items, 2, 128 * kHeadDim * 4, p.tiled ? nullptr : p.split.ws, p.split_ws_bytes);
+  p.items_per_xcd = (p.split.first + kNumXcd - 1) / kNumXcd;
+  p.split.main_wgs = p.items_per_xcd * kNumXcd;
+  const int split_items = p.num_items - p.split.first;
   void (*fn)(const BwdParams) = p.tiled ? &dq_from_ds_kernel<true> : &dq_from_ds_kernel<false>;
   hipError_t e = hipSuccess;
   if (p.tiled && (e = zero_unit_address(&p.zero_unit)) != hipSuccess) return e;
   e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(fn, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
+  hipLaunchKernelGGL(fn, dim3(p.split.main_wgs + split_items * p.split.parts), dim3(256), kSmem, stream, p);
+  if (split_items > 0)
+    return launch_partial_sum(p.split.ws, p.split.parts, 128 * kHeadDim, p.dq, (int64_t)p.split.first * 128, split_items, p.scale, stream);
   return hipGetLastError();
 }
 

@@ -30,6 +30,7 @@ constexpr int kSlab = 32;                      // keys per LDS slab
 constexpr int kSlabBytes = kSlab * kRowBytes;  // 8 KiB
 constexpr int kRing = 4;                       // slabs per ring
 constexpr float kLazy = 8.f;                   // log2 headroom before the softmax reference is raised
+constexpr int kFwdSlotBytes = (128 * kHeadDim + 2 * 128) * 4;  // partial result of one part of a split item
 
 template <int N>
 using IC = std::integral_constant<int, N>;
@@ -125,8 +126,17 @@ __global__ __attribute__((amdgpu_flat_work_group_size(64 * kWaves, 64 * kWaves),
 
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int item = xcd_remap(blockIdx.x, p.items_per_xcd);
-  if (item >= p.num_items) return;
+  // whole items first (dealt to the XCDs in contiguous spans), then the parts of the split items
+  int item, part = 0, parts = 1;
+  if ((int)blockIdx.x < p.split.main_wgs) {
+    item = xcd_remap(blockIdx.x, p.items_per_xcd);
+    if (item >= p.split.first) return;
+  } else {
+    const int s = blockIdx.x - p.split.main_wgs;
+    item = p.split.first + s / p.split.parts;
+    part = s - (item - p.split.first) * p.split.parts;
+    parts = p.split.parts;
+  }
   const int tiles_per_head = p.Sq / TQ;
   const int bh = item / tiles_per_head;
   const int qt = item - bh * tiles_per_head;
@@ -145,7 +155,12 @@ __global__ __attribute__((amdgpu_flat_work_group_size(64 * kWaves, 64 * kWaves),
   // predicate bit of this lane's 16-row group in a tile-list entry
   const int group_bit = 1 << (2 * wave + (l32 >> 4));
   const int nsub = p.k_block / kSlab;
-  const int nsteps = cnt * nsub;
+  // this work-group's range of 32-key steps of the list: all of it, or part `part` of `parts` (even boundaries)
+  const int steps_all = cnt * nsub;
+  const int t_begin = parts == 1 ? 0 : 2 * (int)(((int64_t)(steps_all / 2) * part) / parts);
+  const int t_end = parts == 1 ? steps_all : 2 * (int)(((int64_t)(steps_all / 2) * (part + 1)) / parts);
+  const int nsteps = t_end - t_begin;
+  const int e_begin = t_begin / nsub, sub_begin = t_begin - e_begin * nsub;
 
   FwdState st;
   // Q as the B operand: lane holds row l32, d = 16 ks + 8 h .. +7
@@ -171,9 +186,9 @@ __global__ __attribute__((amdgpu_flat_work_group_size(64 * kWaves, 64 * kWaves),
   // Slab source offsets, in list order.  The list entry of the following key block is read one block ahead, so that
   // the scalar load is off the critical path.  V requests trail K requests by two slabs and reuse their offsets.
   const int64_t block_bytes = (int64_t)p.k_block * kRowBytes;
-  int e_next = 1, rem = nsub;
-  int64_t src_off = cnt > 0 ? key_block(0) * block_bytes : 0;
-  int blk_next = cnt > 1 ? key_block(1) : 0;
+  int e_next = e_begin + 1, rem = nsub - sub_begin;
+  int64_t src_off = nsteps > 0 ? key_block(e_begin) * block_bytes + (int64_t)sub_begin * kSlabBytes : 0;
+  int blk_next = e_next < cnt ? key_block(e_next) : 0;
   auto next_off = [&]() -> int64_t {
     const int64_t off = src_off;
     if (--rem == 0) {
@@ -279,9 +294,25 @@ __global__ __attribute__((amdgpu_flat_work_group_size(64 * kWaves, 64 * kWaves),
     if (w_prev) pv_half(st, v_lds + ((nsteps - 1) & 3) * kSlabBytes, p_prev);
   }
 
+  const float l = sum_halves(st.l_run);
+  if (parts > 1) {
+    // part of a split item: unnormalised O^T, the softmax reference in log2 units and the denominator go to the workspace
+    float* slot = p.split.ws + ((int64_t)(item - p.split.first) * parts + part) * (kFwdSlotBytes / 4);
+    float* prow = slot + (wave * 32 + l32) * kHeadDim;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        *reinterpret_cast<f32x4*>(prow + 32 * mb + 8 * g + 4 * h) =
+            (f32x4){st.acc_o[mb][4 * g + 0], st.acc_o[mb][4 * g + 1], st.acc_o[mb][4 * g + 2], st.acc_o[mb][4 * g + 3]};
+    if (h == 0) {
+      slot[TQ * kHeadDim + wave * 32 + l32] = st.m_run * st.c;
+      slot[TQ * kHeadDim + TQ + wave * 32 + l32] = l;
+    }
+    return;
+  }
   // epilogue: O = O^T / l, LSE = ln2 * (c m + log2 l)
   __bf16* orow = p.o + (qrow0 + l32) * kHeadDim;
-  const float l = sum_halves(st.l_run);
   const float inv = l > 0.f ? 1.f / l : 0.f;
   if (h == 0) p.lse[qrow0 + l32] = l > 0.f ? (st.m_run * st.c + __builtin_log2f(l)) * 0.6931471805599453f : -INFINITY;
 #pragma unroll
@@ -294,16 +325,48 @@ __global__ __attribute__((amdgpu_flat_work_group_size(64 * kWaves, 64 * kWaves),
     }
 }
 
+// Combines the parts of the split items: O = sum_p 2^(m_p - m) O_p / sum_p 2^(m_p - m) l_p with m = max_p m_p, in part
+// order.  One thread per (query row, four head-dim columns).
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void fwd_merge_kernel(const FwdParams p) {
+  const int tid = threadIdx.x;
+  const int row = blockIdx.x * 8 + (tid >> 5), c4 = (tid & 31) * 4;  // row among the 128 * (split items) rows
+  const int it = row >> 7, r = row & 127;
+  const int item = p.split.first + it;
+  const int parts = p.split.parts;
+  const float* slot0 = p.split.ws + (int64_t)it * parts * (kFwdSlotBytes / 4);
+  float m = -INFINITY;
+  for (int q = 0; q < parts; ++q) m = fmaxf(m, slot0[(int64_t)q * (kFwdSlotBytes / 4) + 128 * kHeadDim + r]);
+  float l = 0.f;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int q = 0; q < parts; ++q) {
+    const float* slot = slot0 + (int64_t)q * (kFwdSlotBytes / 4);
+    const float mq = slot[128 * kHeadDim + r];
+    const float w = mq == -INFINITY ? 0.f : fast_exp2(mq - m);
+    l += w * slot[128 * kHeadDim + 128 + r];
+    const f32x4 o4 = *reinterpret_cast<const f32x4*>(slot + r * kHeadDim + c4);
+    acc += w * o4;
+  }
+  const float inv = l > 0.f ? 1.f / l : 0.f;
+  const int64_t orow = (int64_t)item * 128 + r;  // items are consecutive 128-row tiles of [B, Hq, Sq]
+  *reinterpret_cast<bf16x4*>(p.o + orow * kHeadDim + c4) = pack4(acc[0] * inv, acc[1] * inv, acc[2] * inv, acc[3] * inv);
+  if (c4 == 0) p.lse[orow] = l > 0.f ? (m + __builtin_log2f(l)) * 0.6931471805599453f : -INFINITY;
+}
+
 hipError_t launch_fwd(FwdParams p, hipStream_t stream) {
   constexpr int kSmem = 2 * kRing * kSlabBytes;
   const bool wide = !p.tiled && p.q_block % 384 == 0 && p.variant != 1;
   void (*fn)(const FwdParams) = p.tiled ? &fwd_kernel<true, 4> : wide ? &fwd_kernel<false, 12> : &fwd_kernel<false, 4>;
   const int rows = wide ? 384 : 128;
   p.num_items = p.B * p.Hq * (p.Sq / rows);
-  p.items_per_xcd = (p.num_items + kNumXcd - 1) / kNumXcd;
+  // tail splitting for the 128-row kernel on block lists (two work-groups per compute unit)
+  p.split = plan_split(p.num_items, 2, kFwdSlotBytes, (p.tiled || wide) ? nullptr : p.split.ws, p.split_ws_bytes);
+  p.items_per_xcd = (p.split.first + kNumXcd - 1) / kNumXcd;
+  p.split.main_wgs = p.items_per_xcd * kNumXcd;
+  const int split_wgs = (p.num_items - p.split.first) * p.split.parts;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(fn, dim3(p.items_per_xcd * kNumXcd), dim3(rows * 2), kSmem, stream, p);
+  hipLaunchKernelGGL(fn, dim3(p.split.main_wgs + split_wgs), dim3(rows * 2), kSmem, stream, p);
+  if (split_wgs > 0) hipLaunchKernelGGL(fwd_merge_kernel, dim3((p.num_items - p.split.first) * 16), dim3(256), 0, stream, p);
   return hipGetLastError();
 }
 

@@ -22,8 +22,8 @@ struct SplitPlan {
   int main_wgs;   // work-groups in front of the split ones (a multiple of the XCD count)
 };
 
-// Items and work-group slots of a launch -> plan.  `slot_bytes` is what one part stores; the workspace must hold
-// (items - first) * parts of them.
+// Items and work-group slots of a launch -> plan (first = num_items, parts = 1 when nothing is split).  `slot_bytes` is
+// what one part stores; the workspace must hold (num_items - first) * parts of them.  main_wgs is left to the launcher.
 SplitPlan plan_split(int num_items, int wgs_per_cu, int64_t slot_bytes, void* ws, int64_t ws_bytes);
 
 constexpr int kSplitMaxSlots = 512;                           // two work-groups on each of 256 compute units
@@ -45,6 +45,7 @@ struct FwdParams {
   // tiled = 1: q_cnt / q_idx are tile lists (qt_cnt [mask_bh, Sq/128], qt_ent [mask_bh, Sq/128, nK], see
   // tile_lists_kernel) instead of block lists
   int tiled;
+  int64_t split_ws_bytes;  // size of split.ws as handed in by the caller
   int variant;  // 0: 384-row work-groups where q_block allows (measurement of that variant); 1: 128-row work-groups
   SplitPlan split;
 };
@@ -87,6 +88,7 @@ struct BwdParams {
   const int32_t* k_slot;
   const char* zero_unit;
   SplitPlan split;
+  int64_t split_ws_bytes;  // size of split.ws as handed in by the caller
 };
 
 hipError_t launch_mask_compact(const uint8_t* mask, int64_t mask_bh, int nQ, int nK, int32_t* q_cnt, int32_t* q_idx,
@@ -103,7 +105,10 @@ hipError_t launch_fwd(FwdParams p, hipStream_t stream);
 hipError_t launch_bwd_stats(const __bf16* o, const __bf16* d_o, const float* lse, float* stats, int64_t rows, hipStream_t stream);
 hipError_t launch_bwd_dq(BwdParams p, hipStream_t stream);
 hipError_t launch_bwd_dkdv(BwdParams p, hipStream_t stream);
+hipError_t launch_bwd_dkdv64(BwdParams p, hipStream_t stream);  // block lists only: 64 keys per wave, one wave per SIMD
 hipError_t launch_bwd_dq_from_ds(BwdParams p, hipStream_t stream);
+hipError_t launch_partial_sum(const float* ws, int parts, int64_t slot_floats, __bf16* out, int64_t out_row0, int n_items, float scale,
+                              hipStream_t stream);
 hipError_t launch_probe_mfma(const float* src, float* sink, int work_groups, int iters, hipStream_t stream);
 hipError_t launch_pair_slots(const int32_t* q_cnt, const int32_t* q_idx, const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh,
                              int nQ, int nK, int32_t* pair_base, int32_t* q_slot, hipStream_t stream);

@@ -48,14 +48,18 @@ class BlockLists:
     pair_base: Optional[torch.Tensor] = None  # int32; the last entry is the number of listed pairs
     q_slot: Optional[torch.Tensor] = None     # int32
     k_slot: Optional[torch.Tensor] = None     # int32, tile lists only
-    _count: Optional[tuple] = None            # (pinned host copy of pair_base[-1], event recorded after the copy)
+    _count: Optional[tuple] = None            # (pinned host copy of pair_base at head boundaries, event after the copy)
 
-    def listed_pairs(self):
-        """Number of pairs in the lists (sum of k_cnt), read from the host copy that `number_pairs` requested; waits
-        for that copy only, not for work enqueued after it."""
+    def pair_bounds(self):
+        """pair_base at the head boundaries of the mask ([mask_bh + 1] ints, first 0, last = number of listed pairs), read
+        from the host copy that `number_pairs` requested; waits for that copy only, not for work enqueued after it."""
         host, event = self._count
         event.synchronize()
-        return int(host.item())
+        return host.tolist()
+
+    def listed_pairs(self):
+        """Number of pairs in the lists (sum of k_cnt)."""
+        return int(self.pair_bounds()[-1])
 
     def transposed(self):
         """Lists of the transposed mask (query and key roles swapped); no device work.  Block lists only."""
@@ -216,17 +220,34 @@ def _check_lists(lists, q, B, Hq, Sq, Skv, q_block_size, kv_block_size):
                              f"got {tuple(t.shape)} {t.dtype} on {t.device}")
 
 
+# Workspace for tail splitting (see include/fba.h), allocated per call from torch's caching allocator; MiB, 0 switches
+# splitting off, unset: what the library's planner can use at most.
+SPLIT_WORKSPACE_MIB = os.environ.get("FBA_SPLIT_WORKSPACE_MIB")
+
+
+def _split_workspace(device):
+    """(tensor or None, pointer, bytes) of a fresh tail-splitting workspace on `device`."""
+    n = _lib.load().fba_split_workspace_bytes() if SPLIT_WORKSPACE_MIB is None else int(float(SPLIT_WORKSPACE_MIB) * 2 ** 20)
+    if n <= 0:
+        return None, None, 0
+    ws = torch.empty((n,), dtype=torch.uint8, device=device)
+    return ws, _ptr(ws), n
+
+
 def forward_with_lists(q, k, v, q_block_size, kv_block_size, lists):
     """Forward on compacted lists -> (o [B,H,Sq,128] bf16, lse [B,H,Sq,1] fp32)."""
     B, Hq, Hkv, Sq, Skv = _check_qkv(q, k, v)
     _check_lists(lists, q, B, Hq, Sq, Skv, q_block_size, kv_block_size)
     o = torch.empty_like(q)
     lse = torch.empty((B, Hq, Sq, 1), dtype=torch.float32, device=q.device)
+    args = (_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(lists.q_cnt), _ptr(lists.q_idx), lists.mask_bh,
+            B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size)
     with torch.cuda.device(q.device):
-        _lib.call(
-            "fba_fwd_tiled" if lists.tiled else "fba_fwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(lists.q_cnt), _ptr(lists.q_idx), lists.mask_bh,
-            B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size, _stream(),
-        )
+        if lists.tiled:
+            _lib.call("fba_fwd_tiled", *args, _stream())
+        else:
+            _ws, ws_ptr, ws_bytes = _split_workspace(q.device)
+            _lib.call("fba_fwd", *args, ws_ptr, ws_bytes, _stream())
     return o, lse
 
 
@@ -237,7 +258,7 @@ def number_pairs(lists):
     if lists.pair_base is None:
         dev = lists.k_cnt.device
         i32 = dict(dtype=torch.int32, device=dev)
-        host = torch.empty((1,), dtype=torch.int32, pin_memory=True)
+        host = torch.empty((lists.mask_bh + 1,), dtype=torch.int32, pin_memory=True)
         k_slot = None
         with torch.cuda.device(dev):
             if lists.tiled:
@@ -252,32 +273,65 @@ def number_pairs(lists):
                 q_slot = torch.empty((lists.mask_bh, lists.nQ, lists.nK), **i32)
                 _lib.call("fba_pair_slots", _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), lists.mask_bh,
                           lists.nQ, lists.nK, _ptr(pair_base), _ptr(q_slot), _stream())
-            host.copy_(pair_base[-1:], non_blocking=True)
+            host.copy_(pair_base[:: lists.k_cnt.shape[1]], non_blocking=True)  # one entry per head of the mask, and the total
             event = torch.cuda.Event()
             event.record()
         lists.pair_base, lists.q_slot, lists.k_slot, lists._count = pair_base, q_slot, k_slot, (host, event)
     return lists
 
 
-# Largest dS workspace backward may allocate on its own (GiB); beyond it, or when the allocation fails, backward
-# recomputes S and dP in the dQ kernel instead (fba_bwd).
-DS_WORKSPACE_LIMIT_GIB = float(os.environ.get("FBA_DS_WORKSPACE_LIMIT_GIB", "64"))
+# Largest dS workspace backward allocates on its own (GiB).  A backward pass whose selected pairs need more is run in
+# chunks of heads through a workspace within the limit (every head's dS is independent); when not even one kv head
+# fits, or the allocation fails, backward recomputes S and dP in the dQ kernel instead (fba_bwd), which needs no
+# workspace.
+DS_WORKSPACE_LIMIT_GIB = float(os.environ.get("FBA_DS_WORKSPACE_LIMIT_GIB", "8"))
+
+
+def _unit_pairs(lists, B, Hq, Hkv):
+    """Listed pairs of every (batch, kv head): the heads of a GQA group share their kv head's launch."""
+    bounds = number_pairs(lists).pair_bounds()
+    group = Hq // Hkv
+    if lists.mask_bh == 1:
+        return [bounds[-1] * group] * (B * Hkv), bounds
+    return [bounds[(u + 1) * group] - bounds[u * group] for u in range(B * Hkv)], bounds
 
 
 def ds_workspace_bytes(lists, B, Hq, q_block_size, kv_block_size):
-    """(pairs over all heads, bytes of dS workspace) the hand-over backward needs for these lists."""
+    """(pairs over all heads, bytes of dS workspace) the hand-over backward needs for all heads of these lists at once."""
     listed = number_pairs(lists).listed_pairs()
     pairs = listed * (B * Hq if lists.mask_bh == 1 else 1)
     return pairs, pairs * (128 * 128 if lists.tiled else q_block_size * kv_block_size) * 2
 
 
+def plan_head_chunks(unit_pairs, pair_bytes, limit_bytes):
+    """Cuts the (batch, kv head) units into consecutive chunks of equal length whose dS fits `limit_bytes`: as few chunks
+    as the total needs, shortened while some chunk is still too large.  Returns [(first unit, end unit, pairs)], or None
+    when a single unit does not fit."""
+    n = len(unit_pairs)
+    total = sum(unit_pairs) * pair_bytes
+    if total == 0:
+        return [(0, n, 0)]
+    per = -(-n // max(1, -(-total // max(1, limit_bytes)))) if limit_bytes > 0 else 0
+    while per >= 1:
+        chunks = [(u, min(n, u + per), sum(unit_pairs[u: u + per])) for u in range(0, n, per)]
+        if all(c[2] * pair_bytes <= limit_bytes for c in chunks):
+            return chunks
+        per -= 1
+    return None
+
+
+def _offset(t, elements):
+    """Device pointer `elements` elements into tensor t (may point below t for the shifted dS workspace)."""
+    return ctypes.c_void_p(t.data_ptr() + elements * t.element_size())
+
+
 def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists, hand_over=None):
     """Backward on compacted lists -> (dq, dk, dv), bf16, shaped like q, k, v.
 
-    hand_over=True: the key-major kernel stores dS once and dQ is formed from it (fba_bwd_handover or
-    fba_bwd_tiled_handover, ten products per block pair); False: dQ recomputes S and dP (fba_bwd or fba_bwd_tiled,
-    fourteen products, no workspace); None: hand over when the workspace fits DS_WORKSPACE_LIMIT_GIB and can be
-    allocated."""
+    hand_over=None (default): the key-major kernel stores dS once and dQ is formed from it (ten products per block
+    pair instead of fourteen), in chunks of heads through a workspace of at most DS_WORKSPACE_LIMIT_GIB; if not even one
+    kv head fits, as False.  True: the same with one workspace for all heads, whatever its size (fba_bwd_handover /
+    fba_bwd_tiled_handover in one call).  False: dQ recomputes S and dP (fba_bwd or fba_bwd_tiled, no workspace)."""
     B, Hq, Hkv, Sq, Skv = _check_qkv(q, k, v)
     _check_lists(lists, q, B, Hq, Sq, Skv, q_block_size, kv_block_size)
     if do.dtype != torch.bfloat16:
@@ -292,39 +346,60 @@ def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists,
     dq = torch.empty_like(q)
     dk = torch.empty_like(k)
     dv = torch.empty_like(v)
-    stats = torch.empty((2, B, Hq, Sq), dtype=torch.float32, device=q.device)
-    pairs = ws_bytes = 0
-    ds_ws = None
+    pair_bytes = (128 * 128 if lists.tiled else q_block_size * kv_block_size) * 2
+    chunks = ds_ws = None
     if hand_over or hand_over is None:
-        pairs, ws_bytes = ds_workspace_bytes(lists, B, Hq, q_block_size, kv_block_size)
-        if ws_bytes > 0 and (hand_over or ws_bytes <= DS_WORKSPACE_LIMIT_GIB * 2 ** 30):
+        unit_pairs, bounds = _unit_pairs(lists, B, Hq, Hkv)
+        if sum(unit_pairs) > 0:
+            chunks = [(0, B * Hkv, sum(unit_pairs))] if hand_over else plan_head_chunks(unit_pairs, pair_bytes, int(DS_WORKSPACE_LIMIT_GIB * 2 ** 30))
+        if chunks is not None:
             try:
-                ds_ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=q.device)
+                ds_ws = torch.empty((max(c[2] for c in chunks) * pair_bytes,), dtype=torch.uint8, device=q.device)
             except torch.OutOfMemoryError:
                 if hand_over:
                     raise
-    hand_over = ds_ws is not None
+                chunks = None
+    group = Hq // Hkv
+    M = lists.mask_bh
     with torch.cuda.device(q.device):
-        if hand_over and lists.tiled:
-            _lib.call(
-                "fba_bwd_tiled_handover", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), _ptr(ds_ws), ws_bytes,
-                _ptr(dq), _ptr(dk), _ptr(dv), _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx),
-                _ptr(lists.pair_base), _ptr(lists.k_slot), _ptr(lists.q_slot), pairs, lists.mask_bh,
-                B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size, _stream(),
-            )
-        elif hand_over:
-            _lib.call(
-                "fba_bwd_handover", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), _ptr(ds_ws), ws_bytes,
-                _ptr(dq), _ptr(dk), _ptr(dv), _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx),
-                _ptr(lists.pair_base), _ptr(lists.q_slot), pairs, lists.mask_bh,
-                B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size, _stream(),
-            )
-        else:
-            _lib.call(
-                "fba_bwd_tiled" if lists.tiled else "fba_bwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), _ptr(dq), _ptr(dk), _ptr(dv),
-                _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), lists.mask_bh,
-                B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size, _stream(),
-            )
+        _ws, sp_ptr, sp_bytes = (None, None, 0) if lists.tiled else _split_workspace(q.device)
+        if chunks is None:
+            stats = torch.empty((2, B, Hq, Sq), dtype=torch.float32, device=q.device)
+            common = (_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), _ptr(dq), _ptr(dk), _ptr(dv),
+                      _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), M,
+                      B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size)
+            if lists.tiled:
+                _lib.call("fba_bwd_tiled", *common, _stream())
+            else:
+                _lib.call("fba_bwd", *common, sp_ptr, sp_bytes, _stream())
+            return dq, dk, dv
+        # one launch sequence per chunk of kv heads [u0, u1): every pointer moves to the chunk's first head, the chunk is
+        # described as a batch of one, and the workspace pointer is moved back by the pairs of the heads in front of the
+        # chunk, so that the absolute pair numbers of the lists land inside the workspace
+        stats = torch.empty((2, max(c[1] - c[0] for c in chunks) * group * Sq), dtype=torch.float32, device=q.device)
+        n_qt, n_kt = Sq // 128, Skv // 128
+        for u0, u1, pairs in chunks:
+            h0, nh, nu = u0 * group, (u1 - u0) * group, u1 - u0
+            m0 = h0 if M > 1 else 0  # first row of the per-head list tensors
+            qo, ko = h0 * Sq * HEAD_DIM, u0 * Skv * HEAD_DIM
+            ws_ptr = ctypes.c_void_p(ds_ws.data_ptr() - (bounds[h0] * pair_bytes if M > 1 else 0))
+            shape = (nh if M > 1 else 1, 1, nh, nu, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size)
+            if lists.tiled:
+                _lib.call(
+                    "fba_bwd_tiled_handover", _offset(q, qo), _offset(k, ko), _offset(v, ko), _offset(o, qo), _offset(do, qo), _offset(lse, h0 * Sq),
+                    _ptr(stats), ws_ptr, pairs * pair_bytes, _offset(dq, qo), _offset(dk, ko), _offset(dv, ko),
+                    _offset(lists.q_cnt, m0 * n_qt), _offset(lists.q_idx, m0 * n_qt * lists.nK), _offset(lists.k_cnt, m0 * n_kt),
+                    _offset(lists.k_idx, m0 * n_kt * 4 * n_qt), _offset(lists.pair_base, m0 * n_kt), _offset(lists.k_slot, m0 * n_kt * 4 * n_qt),
+                    _offset(lists.q_slot, m0 * n_qt * n_kt), pairs, *shape, _stream(),
+                )
+            else:
+                nQ, nK = lists.nQ, lists.nK
+                _lib.call(
+                    "fba_bwd_handover", _offset(q, qo), _offset(k, ko), _offset(v, ko), _offset(o, qo), _offset(do, qo), _offset(lse, h0 * Sq),
+                    _ptr(stats), ws_ptr, pairs * pair_bytes, _offset(dq, qo), _offset(dk, ko), _offset(dv, ko),
+                    _offset(lists.q_cnt, m0 * nQ), _offset(lists.q_idx, m0 * nQ * nK), _offset(lists.k_cnt, m0 * nK), _offset(lists.k_idx, m0 * nK * nQ),
+                    _offset(lists.pair_base, m0 * nK), _offset(lists.q_slot, m0 * nQ * nK), pairs, *shape, sp_ptr, sp_bytes, _stream(),
+                )
     return dq, dk, dv
 
 

@@ -54,6 +54,20 @@ int32_t fba_mask_compact(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32
                          int32_t* k_cnt, int32_t* k_idx, void* hip_stream);
 
 /*
+ * Tail splitting (no counterpart in the reference).  Work-groups are handed to free compute-unit slots in index order,
+ * so the last (items % slots) 128-row tiles of a launch would run as a partial round with most of the GPU idle; the same
+ * holds for a whole launch with fewer tiles than slots.  Entry points that take `split_ws` cut the lists of those tiles
+ * into up to eight ranges, run each range in a work-group of its own at the end of the grid, store fp32 partial results
+ * into split_ws and combine them in a small second launch, in a fixed order (results stay bit-reproducible).
+ *   split_ws        null (nothing is split), or 16-byte aligned device memory owned by the caller for the duration of
+ *                   the call's work on the stream; its contents before and after are meaningless
+ *   split_ws_bytes  its size; fba_split_workspace_bytes() is what the planner can use at most (a smaller buffer limits
+ *                   the number of ranges, never correctness)
+ * Block lists only: the _tiled entry points do not split.
+ */
+int64_t fba_split_workspace_bytes(void);
+
+/*
  * Forward.  Replaces attn_forward (attn.cpp:29, flex_block_attn_h100.cu:810-1007; kernel :52-318).
  * Writes o (bf16) and lse (fp32, natural log of the row's softmax denominator including the 1/sqrt(128) scale;
  * -inf and o = 0 for a query block with an empty list).  nQ = Sq / q_block, nK = Skv / k_block.
@@ -61,7 +75,8 @@ int32_t fba_mask_compact(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32
  */
 int32_t fba_fwd(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* q_cnt,
                 const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
-                int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+                int32_t head_dim, int32_t q_block, int32_t k_block,
+                void* split_ws, int64_t split_ws_bytes, void* hip_stream);
 
 /*
  * Backward, three stream-ordered launches.  Replaces attn_backward (attn.cpp:30,
@@ -73,7 +88,8 @@ int32_t fba_fwd(const void* q, const void* k, const void* v, void* o, float* lse
 int32_t fba_bwd(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                 float* stats, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
                 const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
-                int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+                int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,
+                void* split_ws, int64_t split_ws_bytes, void* hip_stream);
 
 /* The three stages of fba_bwd, separately (for profiling one kernel at a time); rows = B * Hq * Sq. */
 int32_t fba_bwd_stats(const void* o, const void* d_o, const float* lse, float* stats, int64_t rows, int32_t head_dim,
@@ -83,7 +99,8 @@ int32_t fba_bwd_dq(const void* q, const void* k, const void* v, const void* d_o,
                    int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
 int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,
                      const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
-                     int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+                     int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,
+                     void* split_ws, int64_t split_ws_bytes, void* hip_stream);
 
 /*
  * Backward with dS handed over in memory.  fba_bwd computes S and dP twice, once in the key-major kernel (dK, dV) and
@@ -107,15 +124,18 @@ int32_t fba_bwd_handover(const void* q, const void* k, const void* v, const void
                          void* ds_ws, int64_t ds_ws_bytes, void* dq, void* dk, void* dv, const int32_t* q_cnt, const int32_t* q_idx,
                          const int32_t* k_cnt, const int32_t* k_idx, const int32_t* pair_base, const int32_t* q_slot, int64_t n_pairs,
                          int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim,
-                         int32_t q_block, int32_t k_block, void* hip_stream);
+                         int32_t q_block, int32_t k_block,
+                         void* split_ws, int64_t split_ws_bytes, void* hip_stream);
 /* Its two attention stages separately (after fba_bwd_stats), for profiling one kernel at a time. */
 int32_t fba_bwd_dkdv_handover(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,
                               void* ds_ws, int64_t ds_ws_bytes, const int32_t* k_cnt, const int32_t* k_idx, const int32_t* pair_base,
                               int64_t n_pairs, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
-                              int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+                              int32_t head_dim, int32_t q_block, int32_t k_block,
+                              void* split_ws, int64_t split_ws_bytes, void* hip_stream);
 int32_t fba_bwd_dq_from_ds(const void* k, const void* ds_ws, int64_t ds_ws_bytes, void* dq, const int32_t* q_cnt, const int32_t* q_idx,
                            const int32_t* q_slot, const int32_t* pair_base, int64_t n_pairs, int64_t mask_bh, int32_t B, int32_t Hq,
-                           int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+                           int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,
+                           void* split_ws, int64_t split_ws_bytes, void* hip_stream);
 
 /*
  * fba_bwd without the `stats` argument, for callers that cannot allocate device memory (code under HIP graph capture,

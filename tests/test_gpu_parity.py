@@ -705,3 +705,108 @@ def test_readme_usage_verbatim(oracle, gpu, block_size):
     assert sparse_mask.dtype == torch.bool and sparse_mask.cpu().tolist() == [[False, True], [True, False]]
     want, _ = oracle.c_attention_forward(query.cpu(), key.cpu(), value.cpu(), sparse_mask.cpu(), block_size, block_size)
     _check(oracle, output, want, "o", {})
+
+
+CHUNK_CASES = [
+    # B, Hq, Hkv, Sq, Skv, q_block, k_block, mask dims, density
+    (1, 6, 6, 768, 768, 128, 128, 4, 0.6),
+    (2, 4, 2, 512, 768, 128, 256, 4, 0.5),
+    (1, 6, 3, 768, 768, 384, 384, 2, 0.7),
+    (2, 2, 2, 512, 512, 64, 64, 4, 0.5),
+    (1, 4, 2, 512, 512, 32, 64, 2, 0.6),
+]
+
+
+@pytest.mark.parametrize("cfg", CHUNK_CASES, ids=lambda c: "B%d_Hq%d_Hkv%d_Sq%d_Skv%d_q%d_k%d_m%d_p%s" % c)
+def test_backward_in_head_chunks(oracle, gpu, cfg, monkeypatch):
+    """The default backward hands dS over in chunks of kv heads through a bounded workspace.  With the limit set so low
+    that every kv head is a chunk of its own (and tail splitting off, so that every tile sums in one order), the result
+    must equal the one-workspace hand-over bit for bit: per-head and shared masks, grouped kv heads, batches, block and
+    tile lists.  With the limit below one head's need the call falls back to the recomputing backward."""
+    import flex_block_attn_amd as fba
+    from flex_block_attn_amd import interface
+
+    B, Hq, Hkv, Sq, Skv, qbs, kbs, mdim, density = cfg
+    nQ, nK = Sq // qbs, Skv // kbs
+    g = torch.Generator().manual_seed(Sq + Skv + qbs + Hq)
+    m = (torch.rand((nQ, nK) if mdim == 2 else (B, Hq, nQ, nK), generator=g) < density).to(gpu)
+    q, k, v, do = (t.to(torch.bfloat16).to(gpu) for t in oracle.seeded_qkv(B, Hq, Hkv, Sq, Skv, seed=Sq + kbs + 1))
+    lists = fba.lists_for(m, qbs, kbs)
+    o, lse = fba.forward_with_lists(q, k, v, qbs, kbs, lists)
+    monkeypatch.setattr(interface, "SPLIT_WORKSPACE_MIB", "0")
+    whole = fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists, hand_over=True)
+    unit_pairs, _ = interface._unit_pairs(lists, B, Hq, Hkv)
+    pair_bytes = (128 * 128 if lists.tiled else qbs * kbs) * 2
+    assert max(unit_pairs) > 0
+    monkeypatch.setattr(interface, "DS_WORKSPACE_LIMIT_GIB", max(unit_pairs) * pair_bytes / 2 ** 30)
+    chunks = interface.plan_head_chunks(unit_pairs, pair_bytes, max(unit_pairs) * pair_bytes)
+    assert len(chunks) == B * Hkv or sum(unit_pairs) == max(unit_pairs) * B * Hkv
+    print(f"chunked backward cfg={cfg} chunks={chunks}", flush=True)
+    chunked = fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists)
+    for a, b in zip(chunked, whole):
+        assert torch.equal(a, b)
+    monkeypatch.setattr(interface, "DS_WORKSPACE_LIMIT_GIB", (max(unit_pairs) * pair_bytes - 1) / 2 ** 30)
+    recomputed = fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists)
+    for a, b in zip(recomputed, fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists, hand_over=False)):
+        assert torch.equal(a, b)
+
+
+def test_backward_workspace_stays_within_its_limit(gpu, monkeypatch):
+    """B1 H8 S7680 full attention: all heads at once would need 944 MB of dS; with a 0.25 GiB limit the default backward
+    runs four chunks of two heads and its peak allocation stays below limit + outputs + statistics + splitting workspace."""
+    import flex_block_attn_amd as fba
+    from flex_block_attn_amd import _lib, interface, masks
+
+    B, H, S, bs = 1, 8, 7680, 384
+    g = torch.Generator(device="cpu").manual_seed(17)
+    q, k, v, do = (torch.randn((B, H, S, 128), generator=g).to(torch.bfloat16).to(gpu) for _ in range(4))
+    lists = fba.compact_block_mask(masks.full_block_mask(S // bs, S // bs).to(gpu), with_pair_numbers=True)
+    o, lse = fba.forward_with_lists(q, k, v, bs, bs, lists)
+    want = fba.backward_with_lists(q, k, v, o, lse, do, bs, bs, lists, hand_over=True)
+    limit = 0.25
+    monkeypatch.setattr(interface, "DS_WORKSPACE_LIMIT_GIB", limit)
+    assert interface.ds_workspace_bytes(lists, B, H, bs, bs)[1] > 3 * limit * 2 ** 30
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    before = torch.cuda.memory_allocated()
+    got = fba.backward_with_lists(q, k, v, o, lse, do, bs, bs, lists)
+    torch.cuda.synchronize()
+    peak = torch.cuda.max_memory_allocated() - before
+    outputs = 3 * q.numel() * 2 + 2 * B * H * S * 4
+    assert peak <= limit * 2 ** 30 + outputs + _lib.load().fba_split_workspace_bytes() + (2 << 20), f"peak {peak} bytes"
+    for a, b in zip(got, want):  # launches of two and of eight heads split their last tiles differently: same sums, another order
+        assert (a.float() - b.float()).abs().max().item() <= 2e-2
+
+
+@pytest.mark.parametrize("cfg", [(1, 2, 2, 1536, 1536, 384, 384), (2, 4, 2, 1024, 768, 128, 256), (1, 3, 3, 3072, 3072, 384, 384), (1, 30, 30, 1536, 1536, 384, 384)],
+                         ids=lambda c: "B%d_Hq%d_Hkv%d_Sq%d_Skv%d_q%d_k%d" % c)
+def test_measurement_variants_give_the_same_bits(gpu, cfg, monkeypatch):
+    """The two kernel variants kept for measurement (FBA_FWD_TILE_ROWS=384: forward with 384-row work-groups;
+    FBA_DKDV_KEYS_PER_WAVE=64: dK/dV with 64 keys per wave, one wave per SIMD) do the same arithmetic in the same order as
+    the default kernels: O, LSE, dK, dV and the handed-over dS (seen through dQ) must be bit-equal, with and without tail
+    splitting, on grouped heads and on launches larger than the GPU."""
+    import flex_block_attn_amd as fba
+    from flex_block_attn_amd import interface
+
+    B, Hq, Hkv, Sq, Skv, qbs, kbs = cfg
+    g = torch.Generator(device="cpu").manual_seed(Sq + Hq)
+    q, do = (torch.randn((B, Hq, Sq, 128), generator=g).to(torch.bfloat16).to(gpu) for _ in range(2))
+    k, v = (torch.randn((B, Hkv, Skv, 128), generator=g).to(torch.bfloat16).to(gpu) for _ in range(2))
+    m = (torch.rand((B, Hq, Sq // qbs, Skv // kbs), generator=g) < 0.6).to(gpu)
+    lists = fba.lists_for(m, qbs, kbs)
+    for split in (None, "0"):
+        monkeypatch.setattr(interface, "SPLIT_WORKSPACE_MIB", split)
+        monkeypatch.delenv("FBA_FWD_TILE_ROWS", raising=False)
+        monkeypatch.delenv("FBA_DKDV_KEYS_PER_WAVE", raising=False)
+        o, lse = fba.forward_with_lists(q, k, v, qbs, kbs, lists)
+        base = [fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists, hand_over=h) for h in (True, False)]
+        if qbs % 384 == 0 and split == "0":  # the 384-row forward does not split its tail
+            monkeypatch.setenv("FBA_FWD_TILE_ROWS", "384")
+            o2, lse2 = fba.forward_with_lists(q, k, v, qbs, kbs, lists)
+            assert torch.equal(o, o2) and torch.equal(lse, lse2)
+        monkeypatch.setenv("FBA_DKDV_KEYS_PER_WAVE", "64")
+        for h, want in zip((True, False), base):
+            print(f"variant test cfg={cfg} split={split} hand_over={h}", flush=True)
+            got = fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists, hand_over=h)
+            for a, b in zip(got, want):
+                assert torch.equal(a, b)

@@ -42,11 +42,11 @@ def _fake(addr=0x1000):
 def test_c_abi_argument_validation(lib):
     h = lib.load()
     f = _fake()
-    # fba_fwd(q,k,v,o,lse,q_cnt,q_idx, mask_bh, B,Hq,Hkv,Sq,Skv,D,q_block,k_block, stream)
+    # fba_fwd(q,k,v,o,lse,q_cnt,q_idx, mask_bh, B,Hq,Hkv,Sq,Skv,D,q_block,k_block, split_ws,split_ws_bytes, stream)
     ok_shape = (1, 1, 2, 2, 256, 256, 128, 128, 128)
 
     def fwd(*shape, q=f):
-        return h.fba_fwd(q, f, f, f, f, f, f, *shape, _null())
+        return h.fba_fwd(q, f, f, f, f, f, f, *shape, _null(), 0, _null())
 
     bad = [
         ((1, 1, 2, 2, 256, 256, 64, 128, 128), "head_dim"),
@@ -104,13 +104,17 @@ def test_c_abi_argument_validation(lib):
         lib.call("fba_mask_compact", f, 0, 4, 4, f, f, f, f, _null())
     assert ei.value.code == lib.FBA_ERR_INVALID and "positive" in ei.value.message
     # a 4-D mask is indexed by the QUERY head: with grouped kv heads a mask with one slice per kv head is rejected
-    assert h.fba_fwd(f, f, f, f, f, f, f, 2, 1, 4, 2, 256, 256, 128, 128, 128, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_fwd(f, f, f, f, f, f, f, 2, 1, 4, 2, 256, 256, 128, 128, 128, _null(), 0, _null()) == lib.FBA_ERR_INVALID
     assert b"mask_bh" in h.fba_last_error()
-    assert h.fba_bwd(*([f] * 14), 2, 1, 4, 2, 256, 256, 128, 128, 128, _null()) == lib.FBA_ERR_INVALID and b"mask_bh" in h.fba_last_error()
+    assert h.fba_bwd(*([f] * 14), 2, 1, 4, 2, 256, 256, 128, 128, 128, _null(), 0, _null()) == lib.FBA_ERR_INVALID and b"mask_bh" in h.fba_last_error()
     # backward validates every argument before its first launch: a bad gradient pointer is reported, nothing is enqueued
     bwd_args = [f] * 14
     bwd_args[7] = _null()  # dq
-    assert h.fba_bwd(*bwd_args, 1, 1, 2, 2, 256, 256, 128, 128, 128, _null()) == lib.FBA_ERR_INVALID and b"dq is null" in h.fba_last_error()
+    assert h.fba_bwd(*bwd_args, 1, 1, 2, 2, 256, 256, 128, 128, 128, _null(), 0, _null()) == lib.FBA_ERR_INVALID and b"dq is null" in h.fba_last_error()
+    # the tail-splitting workspace is optional; when given it must be 16-byte aligned with a size that is not negative
+    assert h.fba_fwd(f, f, f, f, f, f, f, *ok_shape, _fake(0x1008), 1 << 20, _null()) == lib.FBA_ERR_INVALID and b"split_ws" in h.fba_last_error()
+    assert h.fba_fwd(f, f, f, f, f, f, f, *ok_shape, f, -1, _null()) == lib.FBA_ERR_INVALID and b"split_ws_bytes" in h.fba_last_error()
+    assert h.fba_split_workspace_bytes() >= 32 * 2 ** 20
 
 
 def test_operator_surface_names():
