@@ -6,8 +6,9 @@ Modes, sweeps and CSV layout follow benchmark/{dynamic/random,static/swa,full}/s
 head, head_dim 128, block 384, seq_len 11520 ... 84480, sparse rates 0.2 ... 0.8 (random_fwd.sh:4-11); one row per
 configuration with the reference's leading columns (batch_size, seq_len, num_heads, head_dim, block_size,
 sparse_rate) and its columns for this operator, `ptm_attn_masks`, `ptm_attn_executes` (forward, ms), `ptm_attn_bwd`
-(backward through autograd, ms) and `ptm_fwd_memory` / `ptm_bwd_memory` (peak bytes), so that rows can be set beside
-the published H800/H20 tables.  Times are means over `--rep` calls measured with HIP events on the launch stream.
+(backward through autograd of the scripts' own loss expression, ms) and `ptm_fwd_memory` / `ptm_bwd_memory` (peak bytes
+allocated, as torch reports them), so that rows can be set beside the published H800/H20 tables.  Times are means over
+`--rep` calls measured with HIP events on the launch stream.
 """
 import argparse
 import csv
@@ -70,7 +71,10 @@ def run_one(mode, batch, seq_len, heads, block_size, sparse_rate, warmup, rep, s
     out = flex_block_attn_func(q, k, v, block_size, block_size, mask)
     torch.cuda.synchronize()
     fwd_mem = torch.cuda.max_memory_allocated()
-    loss = out.sum()
+    # the reference's scripts time backward on this expression (random_bwd.py:114-122): the result in (batch, seq, heads,
+    # dim) layout, made contiguous, summed, squared
+    res = out.transpose(1, 2).contiguous()
+    loss = res.sum() * res.sum()
     bwd_ms = mean_ms(lambda: loss.backward(retain_graph=True), warmup, rep)
     torch.cuda.reset_peak_memory_stats()
     loss.backward(retain_graph=True)

@@ -280,11 +280,19 @@ def number_pairs(lists):
     return lists
 
 
-# Largest dS workspace backward allocates on its own (GiB).  A backward pass whose selected pairs need more is run in
-# chunks of heads through a workspace within the limit (every head's dS is independent); when not even one kv head
-# fits, or the allocation fails, backward recomputes S and dP in the dQ kernel instead (fba_bwd), which needs no
-# workspace.
+# Largest dS workspace backward allocates on its own: at most DS_WORKSPACE_LIMIT_GIB, and at most DS_WORKSPACE_FACTOR
+# times the bytes of the call's own tensors (q, k, v, o, dO, dq, dk, dv), so that backward memory stays proportional to
+# the sequence length like the reference's.  A backward pass whose selected pairs need more is run in chunks of heads
+# through a workspace within the limit (every head's dS is independent); when not even one kv head fits, or the
+# allocation fails, backward recomputes S and dP in the dQ kernel instead (fba_bwd), which needs no workspace.
 DS_WORKSPACE_LIMIT_GIB = float(os.environ.get("FBA_DS_WORKSPACE_LIMIT_GIB", "8"))
+DS_WORKSPACE_FACTOR = float(os.environ.get("FBA_DS_WORKSPACE_FACTOR", "6"))
+
+
+def ds_workspace_limit(q, k):
+    """Bytes of dS workspace the default backward may allocate for these q and k/v shapes."""
+    own = (5 * q.numel() + 4 * k.numel()) * 2  # q, o, dO, dq and k, v, dk, dv (bf16)
+    return int(min(DS_WORKSPACE_LIMIT_GIB * 2 ** 30, DS_WORKSPACE_FACTOR * own))
 
 
 def _unit_pairs(lists, B, Hq, Hkv):
@@ -329,8 +337,8 @@ def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists,
     """Backward on compacted lists -> (dq, dk, dv), bf16, shaped like q, k, v.
 
     hand_over=None (default): the key-major kernel stores dS once and dQ is formed from it (ten products per block
-    pair instead of fourteen), in chunks of heads through a workspace of at most DS_WORKSPACE_LIMIT_GIB; if not even one
-    kv head fits, as False.  True: the same with one workspace for all heads, whatever its size (fba_bwd_handover /
+    pair instead of fourteen), in chunks of heads through a workspace of at most `ds_workspace_limit(q, k)` bytes; if not
+    even one kv head fits, as False.  True: the same with one workspace for all heads, whatever its size (fba_bwd_handover /
     fba_bwd_tiled_handover in one call).  False: dQ recomputes S and dP (fba_bwd or fba_bwd_tiled, no workspace)."""
     B, Hq, Hkv, Sq, Skv = _check_qkv(q, k, v)
     _check_lists(lists, q, B, Hq, Sq, Skv, q_block_size, kv_block_size)
@@ -351,7 +359,7 @@ def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists,
     if hand_over or hand_over is None:
         unit_pairs, bounds = _unit_pairs(lists, B, Hq, Hkv)
         if sum(unit_pairs) > 0:
-            chunks = [(0, B * Hkv, sum(unit_pairs))] if hand_over else plan_head_chunks(unit_pairs, pair_bytes, int(DS_WORKSPACE_LIMIT_GIB * 2 ** 30))
+            chunks = [(0, B * Hkv, sum(unit_pairs))] if hand_over else plan_head_chunks(unit_pairs, pair_bytes, ds_workspace_limit(q, k))
         if chunks is not None:
             try:
                 ds_ws = torch.empty((max(c[2] for c in chunks) * pair_bytes,), dtype=torch.uint8, device=q.device)

@@ -601,6 +601,7 @@ def test_backward_falls_back_without_workspace(gpu, monkeypatch):
     o, lse = fba.forward_with_lists(q, k, v, 128, 128, lists)
     want = fba.backward_with_lists(q, k, v, o, lse, do, 128, 128, lists, hand_over=False)
     monkeypatch.setattr(interface, "DS_WORKSPACE_LIMIT_GIB", 0.0)
+    assert interface.ds_workspace_limit(q, k) == 0
     got = fba.backward_with_lists(q, k, v, o, lse, do, 128, 128, lists)
     for a, b in zip(got, want):
         assert torch.equal(a, b)
@@ -738,6 +739,7 @@ def test_backward_in_head_chunks(oracle, gpu, cfg, monkeypatch):
     unit_pairs, _ = interface._unit_pairs(lists, B, Hq, Hkv)
     pair_bytes = (128 * 128 if lists.tiled else qbs * kbs) * 2
     assert max(unit_pairs) > 0
+    monkeypatch.setattr(interface, "DS_WORKSPACE_FACTOR", 1e9)  # only the absolute limit counts here
     monkeypatch.setattr(interface, "DS_WORKSPACE_LIMIT_GIB", max(unit_pairs) * pair_bytes / 2 ** 30)
     chunks = interface.plan_head_chunks(unit_pairs, pair_bytes, max(unit_pairs) * pair_bytes)
     assert len(chunks) == B * Hkv or sum(unit_pairs) == max(unit_pairs) * B * Hkv
@@ -764,6 +766,7 @@ def test_backward_workspace_stays_within_its_limit(gpu, monkeypatch):
     o, lse = fba.forward_with_lists(q, k, v, bs, bs, lists)
     want = fba.backward_with_lists(q, k, v, o, lse, do, bs, bs, lists, hand_over=True)
     limit = 0.25
+    monkeypatch.setattr(interface, "DS_WORKSPACE_FACTOR", 1e9)
     monkeypatch.setattr(interface, "DS_WORKSPACE_LIMIT_GIB", limit)
     assert interface.ds_workspace_bytes(lists, B, H, bs, bs)[1] > 3 * limit * 2 ** 30
     torch.cuda.synchronize()
@@ -810,3 +813,26 @@ def test_measurement_variants_give_the_same_bits(gpu, cfg, monkeypatch):
             got = fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists, hand_over=h)
             for a, b in zip(got, want):
                 assert torch.equal(a, b)
+
+
+def test_backward_memory_follows_the_sequence_length(gpu):
+    """One head, S=30720, all 80 x 80 blocks of 384: the dS of that head (1.9 GB) is more than the default backward may
+    allocate (six times the call's own tensors), so it recomputes instead and its peak allocation stays within twice the
+    144.8 MB the reference's backward needs for the same problem (benchmark/full/results/full_memory_results_384.csv:4,
+    column ptm_bwd_memory); forward + backward of the operator through autograd."""
+    import flex_block_attn_amd as fba
+    from flex_block_attn_amd import masks
+
+    S, bs = 30720, 384
+    g = torch.Generator(device="cpu").manual_seed(23)
+    q, k, v = (torch.randn((1, 1, S, 128), generator=g).to(torch.bfloat16).to(gpu).requires_grad_(True) for _ in range(3))
+    m = masks.full_block_mask(S // bs, S // bs).to(gpu)
+    torch.cuda.synchronize()
+    torch.cuda.reset_peak_memory_stats()
+    before = torch.cuda.memory_allocated()
+    o = fba.flex_block_attn_func(q, k, v, bs, bs, m)
+    o.sum().backward()
+    torch.cuda.synchronize()
+    peak = torch.cuda.max_memory_allocated() - before + 3 * q.numel() * 2  # the reference's figure counts q, k, v too
+    assert peak <= 2 * 144.8e6, f"peak {peak * 1e-6:.1f} MB"
+    assert torch.isfinite(q.grad).all() and torch.isfinite(k.grad).all() and torch.isfinite(v.grad).all()
