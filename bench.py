@@ -255,7 +255,7 @@ def main():
         "fwd": lambda: _lib.call("fba_fwd", _ptr(q), _ptr(k), _ptr(v), _ptr(o2), _ptr(lse2), _ptr(lists.q_cnt), _ptr(lists.q_idx), *common, sp_ptr, sp_bytes, _stream()),
         "bwd_stats": lambda: _lib.call("fba_bwd_stats", _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), B * H * S, D, _stream()),
         "bwd_dkdv": lambda: _lib.call("fba_bwd_dkdv", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(stats), _ptr(dk), _ptr(dv), _ptr(lists.k_cnt), _ptr(lists.k_idx), *common, sp_ptr, sp_bytes, _stream()),
-        "bwd_dq": lambda: _lib.call("fba_bwd_dq", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(stats), _ptr(dq), _ptr(lists.q_cnt), _ptr(lists.q_idx), *common, _stream()),
+        "bwd_dq": lambda: _lib.call("fba_bwd_dq", _ptr(q), _ptr(k), _ptr(v), _ptr(do), _ptr(stats), _ptr(dq), _ptr(lists.q_cnt), _ptr(lists.q_idx), *common, sp_ptr, sp_bytes, _stream()),
     }
     if mask_fn:
         q_mean, k_mean = fba.block_mean(q, qbs), fba.block_mean(k, kbs)

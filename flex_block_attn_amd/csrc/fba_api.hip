@@ -54,11 +54,14 @@ int check_ptrs(std::initializer_list<std::pair<const char*, const void*>> ps) {
   return FBA_OK;
 }
 
-// Which dK/dV kernel runs on block lists: the one with 32 keys per wave (two waves per SIMD), or, when the environment
-// asks for it (measurement of that variant), the one with 64 keys per wave (one wave per SIMD).
+// Which dK/dV kernel runs on block lists.  Without the dS hand-over the kernel with 64 keys per wave (one wave per SIMD)
+// is the faster one (7-11 % on every shape measured); with it the kernel with 32 keys per wave (two waves per SIMD) is,
+// because a wave alone on its SIMD pays for every cycle its dS stores take to issue.  Both do the same arithmetic in the
+// same order.  FBA_DKDV_KEYS_PER_WAVE = 32 or 64 overrides the choice (measurement of the two variants).
 hipError_t launch_dkdv_variant(fba::BwdParams& p, hipStream_t stream) {
-  const char* keys = getenv("FBA_DKDV_KEYS_PER_WAVE");
-  if (!p.tiled && keys && atoi(keys) == 64) return fba::launch_bwd_dkdv64(p, stream);
+  const char* env = getenv("FBA_DKDV_KEYS_PER_WAVE");
+  const int keys = env ? atoi(env) : (p.ds_ws == nullptr ? 64 : 32);
+  if (!p.tiled && keys == 64) return fba::launch_bwd_dkdv64(p, stream);
   return fba::launch_bwd_dkdv(p, stream);
 }
 
@@ -227,17 +230,20 @@ int32_t fba_bwd_stats(const void* o, const void* d_o, const float* lse, float* s
 
 static int dq_impl(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dq,
                    const int32_t* q_cnt, const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
-                   int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream, bool tiled) {
+                   int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* split_ws, int64_t split_ws_bytes,
+                   void* hip_stream, bool tiled) {
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"d_o", d_o}, {"dq", dq}})) return rc;
   if (!stats || !q_cnt || !q_idx) return fail(FBA_ERR_INVALID, "null pointer argument");
   if (int rc = check_lists(s, tiled, "dq")) return rc;
+  if (int rc = check_split_ws(split_ws, split_ws_bytes)) return rc;
   fba::BwdParams p{};
   fill_bwd(p, s);
   p.tiled = tiled ? 1 : 0;
   p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.d_o = (const __bf16*)d_o;
   p.stats = stats; p.dq = (__bf16*)dq; p.q_cnt = q_cnt; p.q_idx = q_idx;
+  p.split.ws = (float*)split_ws; p.split_ws_bytes = split_ws_bytes;
   hipError_t e = fba::launch_bwd_dq(p, (hipStream_t)hip_stream);
   return e == hipSuccess ? FBA_OK : hip_fail(e, "dq launch");
 }
@@ -280,13 +286,16 @@ static int bwd_impl(const void* q, const void* k, const void* v, const void* o, 
   if (int rc = dkdv_impl(q, k, v, d_o, stats, dk, dv, k_cnt, k_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block,
                          split_ws, split_ws_bytes, hip_stream, tiled))
     return rc;
-  return dq_impl(q, k, v, d_o, stats, dq, q_cnt, q_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream, tiled);
+  return dq_impl(q, k, v, d_o, stats, dq, q_cnt, q_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, split_ws, split_ws_bytes,
+                 hip_stream, tiled);
 }
 
 int32_t fba_bwd_dq(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dq,
                    const int32_t* q_cnt, const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
-                   int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
-  return dq_impl(q, k, v, d_o, stats, dq, q_cnt, q_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, hip_stream, false);
+                   int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* split_ws, int64_t split_ws_bytes,
+                   void* hip_stream) {
+  return dq_impl(q, k, v, d_o, stats, dq, q_cnt, q_idx, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, split_ws, split_ws_bytes,
+                 hip_stream, false);
 }
 
 int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,

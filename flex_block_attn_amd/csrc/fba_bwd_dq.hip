@@ -40,8 +40,17 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int item = xcd_remap(blockIdx.x, p.items_per_xcd);
-  if (item >= p.num_items) return;
+  // whole items first (dealt to the XCDs in contiguous spans), then the parts of the split items
+  int item, part = 0, parts = 1;
+  if ((int)blockIdx.x < p.split.main_wgs) {
+    item = xcd_remap(blockIdx.x, p.items_per_xcd);
+    if (item >= p.split.first) return;
+  } else {
+    const int s = blockIdx.x - p.split.main_wgs;
+    item = p.split.first + s / p.split.parts;
+    part = s - (item - p.split.first) * p.split.parts;
+    parts = p.split.parts;
+  }
   const int tiles_per_head = p.Sq / TQ;
   const int bh = item / tiles_per_head;
   const int qt = item - bh * tiles_per_head;
@@ -59,7 +68,11 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   const int group_bit = 1 << (2 * wave + (l32 >> 4));  // this lane's 16-row group in a tile-list entry
   const int wave_bits = 3 << (2 * wave);               // both groups of this wave
   const int nsub = p.k_block / kSlab;
-  const int nsteps = cnt * nsub;
+  // this work-group's range of 32-key steps of the list: all of it, or part `part` of `parts` (even boundaries)
+  const int steps_all = cnt * nsub;
+  const int t_begin = parts == 1 ? 0 : 2 * (int)(((int64_t)(steps_all / 2) * part) / parts);
+  const int nsteps = (parts == 1 ? steps_all : 2 * (int)(((int64_t)(steps_all / 2) * (part + 1)) / parts)) - t_begin;
+  const int e_begin = t_begin / nsub, sub_begin = t_begin - e_begin * nsub;
 
   // Q and dO as B operands: lane holds row l32, d = 16 ks + 8 h .. +7
   bf16x8 qreg[8], doreg[8];
@@ -89,9 +102,9 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 
   // slab source offsets in list order; the list entry of the following key block is read one block ahead
   const int64_t block_bytes = (int64_t)p.k_block * kRowBytes;
-  int e_next = 1, rem = nsub;
-  int64_t src_off = cnt > 0 ? key_block(0) * block_bytes : 0;
-  int blk_next = cnt > 1 ? key_block(1) : 0;
+  int e_next = e_begin + 1, rem = nsub - sub_begin;
+  int64_t src_off = nsteps > 0 ? key_block(e_begin) * block_bytes + (int64_t)sub_begin * kSlabBytes : 0;
+  int blk_next = e_next < cnt ? key_block(e_next) : 0;
   auto copy_next = [&](int ring) {
     dma.copy(ring_dst + ring * kPairBytes, kp + src_off);
     dma.copy(ring_dst + ring * kPairBytes + kSlabBytes, vp + src_off);
@@ -178,6 +191,15 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     }
   }
 
+  if (parts > 1) {  // part of a split item: unscaled fp32 partial sums go to the workspace
+    float* prow = p.split.ws + ((int64_t)(item - p.split.first) * parts + part) * (TQ * kHeadDim) + (wave * 32 + l32) * kHeadDim;
+#pragma unroll
+    for (int mb = 0; mb < 4; ++mb)
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+        *reinterpret_cast<f32x4*>(prow + 32 * mb + 8 * g + 4 * h) = (f32x4){acc[mb][4 * g + 0], acc[mb][4 * g + 1], acc[mb][4 * g + 2], acc[mb][4 * g + 3]};
+    return;
+  }
   __bf16* orow = p.dq + (qrow0 + l32) * kHeadDim;
 #pragma unroll
   for (int mb = 0; mb < 4; ++mb)
@@ -192,14 +214,17 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 hipError_t launch_bwd_dq(BwdParams p, hipStream_t stream) {
   constexpr int kSmem = kRing * kPairBytes;
   p.num_items = p.B * p.Hq * (p.Sq / 128);
-  p.items_per_xcd = (p.num_items + kNumXcd - 1) / kNumXcd;
-  const void* fn = p.tiled ? reinterpret_cast<const void*>(&dq_kernel<true>) : reinterpret_cast<const void*>(&dq_kernel<false>);
-  hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
+  // tail splitting on block lists (two work-groups per compute unit); a part stores a 128 x 128 fp32 tile
+  p.split = plan_split(p.num_items, 2, 128 * kHeadDim * 4, p.tiled ? nullptr : p.split.ws, p.split_ws_bytes);
+  p.items_per_xcd = (p.split.first + kNumXcd - 1) / kNumXcd;
+  p.split.main_wgs = p.items_per_xcd * kNumXcd;
+  const int split_items = p.num_items - p.split.first;
+  void (*fn)(const BwdParams) = p.tiled ? &dq_kernel<true> : &dq_kernel<false>;
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
   if (e != hipSuccess) return e;
-  if (p.tiled)
-    hipLaunchKernelGGL(dq_kernel<true>, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
-  else
-    hipLaunchKernelGGL(dq_kernel<false>, dim3(p.items_per_xcd * kNumXcd), dim3(256), kSmem, stream, p);
+  hipLaunchKernelGGL(fn, dim3(p.split.main_wgs + split_items * p.split.parts), dim3(256), kSmem, stream, p);
+  if (split_items > 0)
+    return launch_partial_sum(p.split.ws, p.split.parts, 128 * kHeadDim, p.dq, (int64_t)p.split.first * 128, split_items, p.scale, stream);
   return hipGetLastError();
 }
 

@@ -96,7 +96,8 @@ int32_t fba_bwd_stats(const void* o, const void* d_o, const float* lse, float* s
                       void* hip_stream);
 int32_t fba_bwd_dq(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dq,
                    const int32_t* q_cnt, const int32_t* q_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
-                   int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+                   int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,
+                   void* split_ws, int64_t split_ws_bytes, void* hip_stream);
 int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_o, const float* stats, void* dk, void* dv,
                      const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
                      int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,

@@ -784,9 +784,9 @@ def test_backward_workspace_stays_within_its_limit(gpu, monkeypatch):
 @pytest.mark.parametrize("cfg", [(1, 2, 2, 1536, 1536, 384, 384), (2, 4, 2, 1024, 768, 128, 256), (1, 3, 3, 3072, 3072, 384, 384), (1, 30, 30, 1536, 1536, 384, 384)],
                          ids=lambda c: "B%d_Hq%d_Hkv%d_Sq%d_Skv%d_q%d_k%d" % c)
 def test_measurement_variants_give_the_same_bits(gpu, cfg, monkeypatch):
-    """The two kernel variants kept for measurement (FBA_FWD_TILE_ROWS=384: forward with 384-row work-groups;
-    FBA_DKDV_KEYS_PER_WAVE=64: dK/dV with 64 keys per wave, one wave per SIMD) do the same arithmetic in the same order as
-    the default kernels: O, LSE, dK, dV and the handed-over dS (seen through dQ) must be bit-equal, with and without tail
+    """The forward variant kept for measurement (FBA_FWD_TILE_ROWS=384: 384-row work-groups) and the two dK/dV kernels
+    (FBA_DKDV_KEYS_PER_WAVE=32 / 64: two waves per SIMD with 32 keys each, the default with the dS hand-over, or one wave
+    per SIMD with 64 keys, the default without) do the same arithmetic in the same order: O, LSE, dK, dV and the handed-over dS (seen through dQ) must be bit-equal, with and without tail
     splitting, on grouped heads and on launches larger than the GPU."""
     import flex_block_attn_amd as fba
     from flex_block_attn_amd import interface
@@ -800,7 +800,7 @@ def test_measurement_variants_give_the_same_bits(gpu, cfg, monkeypatch):
     for split in (None, "0"):
         monkeypatch.setattr(interface, "SPLIT_WORKSPACE_MIB", split)
         monkeypatch.delenv("FBA_FWD_TILE_ROWS", raising=False)
-        monkeypatch.delenv("FBA_DKDV_KEYS_PER_WAVE", raising=False)
+        monkeypatch.setenv("FBA_DKDV_KEYS_PER_WAVE", "32")
         o, lse = fba.forward_with_lists(q, k, v, qbs, kbs, lists)
         base = [fba.backward_with_lists(q, k, v, o, lse, do, qbs, kbs, lists, hand_over=h) for h in (True, False)]
         if qbs % 384 == 0 and split == "0":  # the 384-row forward does not split its tail
