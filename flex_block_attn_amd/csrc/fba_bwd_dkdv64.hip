@@ -521,8 +521,7 @@ hipError_t launch_bwd_dkdv64(BwdParams p, hipStream_t stream) {
   p.num_items = p.B * p.Hkv * (p.Skv / 128);
   // tail splitting (one work-group per compute unit); a part stores two 128 x 128 fp32 tiles
   p.split = plan_split(p.num_items, 1, 2 * 128 * kHeadDim * 4, p.split.ws, p.split_ws_bytes);
-  p.items_per_xcd = (p.split.first + kNumXcd - 1) / kNumXcd;
-  p.split.main_wgs = p.items_per_xcd * kNumXcd;
+  plan_xcd_mapping(p.B * p.Hkv, p.split.first, p.items_per_xcd, p.split.main_wgs);
   const int split_items = p.num_items - p.split.first;
   void (*fn)(const BwdParams) = p.ds_ws != nullptr ? &dkdv64_kernel<true> : &dkdv64_kernel<false>;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);

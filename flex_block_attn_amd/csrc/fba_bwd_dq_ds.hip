@@ -272,8 +272,7 @@ hipError_t launch_bwd_dq_from_ds(BwdParams p, hipStream_t stream) {
   p.num_items = p.B * p.Hq * (p.Sq / 128);
   // tail splitting on block lists (two work-groups per compute unit); a part stores a 128 x 128 fp32 tile
   p.split = plan_split(p.num_items, 2, 128 * kHeadDim * 4, p.tiled ? nullptr : p.split.ws, p.split_ws_bytes);
-  p.items_per_xcd = (p.split.first + kNumXcd - 1) / kNumXcd;
-  p.split.main_wgs = p.items_per_xcd * kNumXcd;
+  plan_xcd_mapping(p.B * p.Hq, p.split.first, p.items_per_xcd, p.split.main_wgs);
   const int split_items = p.num_items - p.split.first;
   void (*fn)(const BwdParams) = p.tiled ? &dq_from_ds_kernel<true> : &dq_from_ds_kernel<false>;
   hipError_t e = hipSuccess;

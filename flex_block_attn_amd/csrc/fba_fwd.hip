@@ -360,8 +360,7 @@ hipError_t launch_fwd(FwdParams p, hipStream_t stream) {
   p.num_items = p.B * p.Hq * (p.Sq / rows);
   // tail splitting for the 128-row kernel on block lists (two work-groups per compute unit)
   p.split = plan_split(p.num_items, 2, kFwdSlotBytes, (p.tiled || wide) ? nullptr : p.split.ws, p.split_ws_bytes);
-  p.items_per_xcd = (p.split.first + kNumXcd - 1) / kNumXcd;
-  p.split.main_wgs = p.items_per_xcd * kNumXcd;
+  plan_xcd_mapping(p.B * p.Hq, p.split.first, p.items_per_xcd, p.split.main_wgs);
   const int split_wgs = (p.num_items - p.split.first) * p.split.parts;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
   if (e != hipSuccess) return e;

@@ -26,6 +26,20 @@ struct SplitPlan {
 // what one part stores; the workspace must hold (num_items - first) * parts of them.  main_wgs is left to the launcher.
 SplitPlan plan_split(int num_items, int wgs_per_cu, int64_t slot_bytes, void* ws, int64_t ws_bytes);
 
+// How the whole items of a launch are dealt to the XCDs (see xcd_remap): contiguous spans when the launch has at least
+// one (batch, head) per XCD, work-group order otherwise.  Sets items_per_xcd and the number of work-groups that come
+// before the split ones.
+inline void plan_xcd_mapping(int heads, int whole_items, int& items_per_xcd, int& main_wgs) {
+  constexpr int kXcds = 8;
+  if (heads >= kXcds) {
+    items_per_xcd = (whole_items + kXcds - 1) / kXcds;
+    main_wgs = items_per_xcd * kXcds;
+  } else {
+    items_per_xcd = 0;
+    main_wgs = whole_items;
+  }
+}
+
 constexpr int kSplitMaxSlots = 512;                           // two work-groups on each of 256 compute units
 constexpr int64_t kSplitSlotBytes = 128 * 128 * 4 * 2;        // dK and dV partials of a key tile; forward: O^T + (m, l)
 constexpr int64_t kSplitWsBytes = (kSplitMaxSlots / 2) * kSplitSlotBytes + (1 << 20);
