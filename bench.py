@@ -241,6 +241,13 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     value = (fl_fwd + fl_bwd) / (ms_per_step * 1e-3) * 1e-12
+    # peak memory of one step above what is resident before it (q, k, v, dO, mask): outputs, lists, statistics, the dS
+    # workspace of the chunked hand-over, the tail-splitting workspace
+    torch.cuda.reset_peak_memory_stats()
+    resident = torch.cuda.memory_allocated()
+    step()
+    torch.cuda.synchronize()
+    step_peak_bytes = torch.cuda.max_memory_allocated() - resident
 
     # ---- per-kernel timing with HIP events on the launch stream -------------------------------------------
     lists = fba.compact_block_mask(mask)
@@ -316,6 +323,7 @@ def main():
         "bwd_ms": bwd_ms, "bwd_TFLOP/s": fl_bwd / (bwd_ms * 1e-3) * 1e-12,
         "bwd_path": "dS hand-over (fba_bwd_handover)" if hand_over else "recompute (fba_bwd)",
         "bwd_recompute_ms": bwd_recompute_ms, "ds_workspace_GB": ws_bytes * 1e-9,
+        "step_peak_memory_GB": step_peak_bytes * 1e-9, "step_ds_workspace_limit_GB": interface.ds_workspace_limit(q, k) * 1e-9,
         "fwd+bwd_kernels_TFLOP/s": (fl_fwd + fl_bwd) / ((bwd_ms + kms["fwd"]["mean_ms"]) * 1e-3) * 1e-12,
         "frac_of_bf16_peak": value / PEAK_BF16_TFLOPS,
         "kernels_ms": {n: kms[n]["mean_ms"] for n in kms},

@@ -79,7 +79,7 @@ int check_split_ws(const void* ws, int64_t bytes) {
 
 extern "C" {
 
-int32_t fba_version(void) { return 1000; }
+int32_t fba_version(void) { return 2000; }
 
 const char* fba_last_error(void) { return g_err; }
 

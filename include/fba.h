@@ -116,7 +116,12 @@ int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_
  *                    (-1 beyond q_cnt).
  *   ds_ws            n_pairs * q_block * k_block bf16, 16-byte aligned; n_pairs = selected pairs over all (batch,
  *                    head): the sum of k_cnt, times B * Hq when mask_bh == 1.  ds_ws_bytes is its size; the caller
- *                    vouches that n_pairs matches the lists (they live in device memory and are not read back).
+ *                    vouches that n_pairs matches the lists (they live in device memory and are not read back): the
+ *                    kernels address ds_ws by the pair numbers in pair_base / q_slot, so lists that do not belong to
+ *                    this n_pairs and workspace make them write out of bounds.
+ * Every head's dS is independent: a caller short of memory may run these entry points once per group of kv heads through
+ * one smaller workspace, with all pointers moved to the group's first head (B = 1) and ds_ws moved back by the pairs in
+ * front of the group when the mask is per head (the pair numbers in the lists are absolute).
  * Other arguments as fba_bwd; dq, dk, dv agree with fba_bwd's to within bf16 rounding of dS (dk, dv bit for bit).
  */
 int32_t fba_pair_slots(const int32_t* q_cnt, const int32_t* q_idx, const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh,
@@ -139,8 +144,8 @@ int32_t fba_bwd_dq_from_ds(const void* k, const void* ds_ws, int64_t ds_ws_bytes
                            void* split_ws, int64_t split_ws_bytes, void* hip_stream);
 
 /*
- * fba_bwd without the `stats` argument, for callers that cannot allocate device memory (code under HIP graph capture,
- * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference, whose host launcher
+ * fba_bwd without the `stats` argument, for callers that cannot allocate device memory (tight serving loops, harnesses
+ * that forbid hipMalloc).  It has no counterpart in the reference, whose host launcher
  * allocates with torch (flex_block_attn_h100.cu:1077-1093).  The statistics live in a 32 MiB array that is part of the
  * library's device image, so the call allocates and frees nothing; it serves up to 4 194 304 query rows
  * (B * Hq * Sq <= 2^22) and returns FBA_ERR_UNSUPPORTED beyond that.  Every call on a GPU uses that GPU's one array:
