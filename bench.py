@@ -12,6 +12,7 @@ Prints ONE JSON line on stdout (everything else goes to stderr).
 """
 import argparse
 import ctypes
+import gc
 import json
 import os
 import statistics
@@ -235,11 +236,16 @@ def main():
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
+    # Python's cyclic garbage collector is kept out of the timed region, as timeit does: a full pass over a process with
+    # torch loaded takes about 40 ms (two steps) and says nothing about the GPU path
+    gc.collect()
+    gc.disable()
     t0 = time.perf_counter()
     for _ in range(args.steps):
         step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    gc.enable()
     value = (fl_fwd + fl_bwd) / (ms_per_step * 1e-3) * 1e-12
     # peak memory of one step above what is resident before it (q, k, v, dO, mask): outputs, lists, statistics, the dS
     # workspace of the chunked hand-over, the tail-splitting workspace

@@ -284,8 +284,13 @@ def number_pairs(lists):
 # times the bytes of the call's own tensors (q, k, v, o, dO, dq, dk, dv), so that backward memory stays proportional to
 # the sequence length like the reference's.  A backward pass whose selected pairs need more is run in chunks of heads
 # through a workspace within the limit (every head's dS is independent); when not even one kv head fits, or the
-# allocation fails, backward recomputes S and dP in the dQ kernel instead (fba_bwd), which needs no workspace.
-DS_WORKSPACE_LIMIT_GIB = float(os.environ.get("FBA_DS_WORKSPACE_LIMIT_GIB", "8"))
+# allocation fails, backward recomputes S and dP in the dQ kernel instead (fba_bwd), which needs no workspace.  The
+# default of 20 GiB lets the benchmark shapes with 24 heads run in chunks of at least 8 heads, one per XCD (chunks of
+# fewer heads are slower per head); FBA_DS_WORKSPACE_LIMIT_GIB=8 costs them up to 9 % of backward.
+# (The limit deliberately reads no allocator or driver state: hipMemGetInfo takes milliseconds, and torch's memory
+# counters build a dictionary of a few hundred entries per call, enough to trigger a full pass of Python's cyclic garbage
+# collector, 40 ms in a process that has torch loaded, every few dozen calls.)
+DS_WORKSPACE_LIMIT_GIB = float(os.environ.get("FBA_DS_WORKSPACE_LIMIT_GIB", "20"))
 DS_WORKSPACE_FACTOR = float(os.environ.get("FBA_DS_WORKSPACE_FACTOR", "6"))
 
 
