@@ -316,21 +316,34 @@ def ds_workspace_bytes(lists, B, Hq, q_block_size, kv_block_size):
     return pairs, pairs * (128 * 128 if lists.tiled else q_block_size * kv_block_size) * 2
 
 
+XCDS = 8  # a launch that gives every XCD whole heads of its own runs faster per head than one that makes XCDs share heads
+
+
 def plan_head_chunks(unit_pairs, pair_bytes, limit_bytes):
     """Cuts the (batch, kv head) units into consecutive chunks of equal length whose dS fits `limit_bytes`: as few chunks
-    as the total needs, shortened while some chunk is still too large.  Returns [(first unit, end unit, pairs)], or None
-    when a single unit does not fit."""
+    as the total needs, shortened while some chunk is still too large, and then, if a chunk holds more than one unit per
+    XCD, shortened to a multiple of the XCD count (twelve heads per chunk cost dK/dV 3 % against eight).  Returns
+    [(first unit, end unit, pairs)], or None when a single unit does not fit."""
     n = len(unit_pairs)
     total = sum(unit_pairs) * pair_bytes
     if total == 0:
         return [(0, n, 0)]
+
+    def cut(per):
+        return [(u, min(n, u + per), sum(unit_pairs[u: u + per])) for u in range(0, n, per)]
+
+    def fits(chunks):
+        return all(c[2] * pair_bytes <= limit_bytes for c in chunks)
+
+    limit_bytes = int(limit_bytes)
     per = -(-n // max(1, -(-total // max(1, limit_bytes)))) if limit_bytes > 0 else 0
-    while per >= 1:
-        chunks = [(u, min(n, u + per), sum(unit_pairs[u: u + per])) for u in range(0, n, per)]
-        if all(c[2] * pair_bytes <= limit_bytes for c in chunks):
-            return chunks
+    while per >= 1 and not fits(cut(per)):
         per -= 1
-    return None
+    if per < 1:
+        return None
+    if per < n and per > XCDS and per % XCDS and fits(cut(per - per % XCDS)):
+        per -= per % XCDS
+    return cut(per)
 
 
 def _offset(t, elements):
