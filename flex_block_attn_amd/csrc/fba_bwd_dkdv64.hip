@@ -297,7 +297,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     // S, dP of the slab in the buffer at byte offset `so` against this wave's 64 keys: every Q / dO operand feeds both key
     // groups.  The operands of step ks+1 are requested before the matrix instructions of step ks are issued; the scheduling
     // fences keep the compiler from moving them back next to their use, where the wave would wait for every fetch.
-    auto scores = [&](int so, bool request, uint32_t req_dst, int64_t req_row, char* ds_unit) {
+    auto scores = [&](auto extras_c, int so, uint32_t req_dst, int64_t req_row, char* ds_unit) {
+      constexpr bool kExtras = decltype(extras_c)::value;  // false for the wave's first slab: nothing to copy or store yet
       // accumulator element 4g + e of half-wave h is query row 8g + 4h + e of the slab; dP starts from -delta of its row
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -326,18 +327,17 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
         // matrix instructions: a wave alone on its SIMD pays for every cycle a memory instruction takes to issue
         // (copies first, stores last: the wait before the next barrier then lets the four youngest operations, the stores,
         // stay in flight)
-        if (ks < 4) {
-          if (request) issue_copy_part(2 * ks, req_dst, req_row);
+        if constexpr (kExtras) {
+          if (ks < 4) issue_copy_part(2 * ks, req_dst, req_row);
         }
         dp[0] = mfma32(dof, vf0, dp[0]);
-        if (ks < 4) {
-          if (request) issue_copy_part(2 * ks + 1, req_dst, req_row);
-        } else if (ks == 4) {
-          if (request) issue_copy_part(8, req_dst, req_row);
+        if constexpr (kExtras) {
+          if (ks < 4) issue_copy_part(2 * ks + 1, req_dst, req_row);
+          else if (ks == 4) issue_copy_part(8, req_dst, req_row);
         }
         dp[1] = mfma32(dof, vf1, dp[1]);
-        if constexpr (kHandOver) {
-          if (ks >= 4 && ds_unit != nullptr)
+        if constexpr (kHandOver && kExtras) {
+          if (ks >= 4)  // scores() runs only while the wave has a further slab, so slab t exists and ds_unit is set
             __builtin_nontemporal_store(dsk[(ks >> 1) & 1][ks & 1],
                                         reinterpret_cast<bf16x8*>(ds_unit + ((ks >> 1) & 1) * 4 * kDsUnitBytes + ((ks & 1) ? ho_off1 : ho_off0)));
         }
@@ -413,7 +413,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
       for (int j = 0; j < 2; ++j)
 #pragma unroll
         for (int e = 0; e < 8; ++e) { pk[grp][j][e] = (__bf16)0.f; dsk[grp][j][e] = (__bf16)0.f; }
-    scores(0, false, 0, 0, nullptr);
+    scores(std::false_type{}, 0, 0, 0, nullptr);
     // Iteration t: slab t lives in buffer t % 3, slab t-1 in (t+2) % 3, slab t+1 in (t+1) % 3.  The first iteration adds
     // nothing (P = dS = 0 against the finite rows of slab 0); the last one, t = nlocal, only adds slab nlocal-1 (its
     // arithmetic runs on stale registers and is dropped), so that every wave passes the same barriers.
@@ -433,16 +433,16 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
       if (kHandOver && stores_in_flight) wait_vmem<4>(); else wait_vmem<0>();
       __syncthreads();  // everybody is done with slab t-1 and everybody's copies of slab t+1 have landed
       const int freed = nxt + kStageBytes == 3 * kStageBytes ? 0 : nxt + kStageBytes;  // buffer of slab t-1 = buffer of slab t+2
-      // slab t+2 replaces slab t-1, if the wave has one; its copies are issued in between the matrix instructions of scores()
+      // slab t+2 replaces slab t-1 (past the end of the lists: a repeat of the last slab that nobody reads); its copies are
+      // issued in between the matrix instructions of scores()
       const int64_t r0 = row_next;
       advance();
       const int64_t r1 = row_next;
       advance();
-      const bool request = t + 2 < nlocal;
       const uint32_t req_dst = ring_dst + 3 * par * kStageBytes + freed;
       stores_in_flight = ds_unit != nullptr;
       if (t + 1 < nlocal) {
-        scores(nxt, request, req_dst, par ? r1 : r0, ds_unit);
+        scores(std::true_type{}, nxt, req_dst, par ? r1 : r0, ds_unit);
       } else if constexpr (kHandOver) {
         if (ds_unit != nullptr) {  // the wave's last slab: no scores() follows that could carry its stores
 #pragma unroll
