@@ -158,30 +158,71 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 #pragma unroll
         for (int ks = 0; ks < 8; ++ks) kreg[grp][ks] = *reinterpret_cast<const bf16x8*>(kp + grp * 32 * kHeadDim + 16 * ks);
     }
-    // Cursor over (query head of the group, list entry, slab): first query row of the next slab to request.
+    // Cursor over (query head of the group, list entry, pair of slabs).  Slabs are numbered in list order; slabs 2i and 2i+1
+    // form pair i, the first for the waves of parity 0, the second for those of parity 1.  A pair never straddles two query
+    // blocks (q_block is a multiple of 128 and ranges start on multiples of four slabs), so the cursor moves a pair at a
+    // time: first query row of the next pair, and (hand-over) the byte offset of the dS unit that the pair's first slab and
+    // this wave's first key group own in the workspace.  Requests run two pairs ahead of the arithmetic; the unit offsets
+    // wait in two variables until their slab's dS is stored, so the lists are walked once only.
     const char* qbase = reinterpret_cast<const char*>(p.q);
     const char* dobase = reinterpret_cast<const char*>(p.d_o);
     const char* stbase = reinterpret_cast<const char*>(p.stats);
-    int g_cur = -1, e_cur = -1, cnt_cur = 0, rem = 1;
-    bool more = true;  // false once every listed slab has been requested; row_next then stays on the last one
+    const int64_t pair_bytes = (int64_t)p.q_block * p.k_block * 2;
+    const int nsub_k = p.k_block / kSlab;
+    const int t_key = 4 * ((kt * TK - kblk * p.k_block) / TK) + 2 * kg;  // this wave's first 32-key slab inside the key block
+    const int ho_off0 = ds_unit_store_off(0, lane), ho_off1 = ds_unit_store_off(1, lane);
+    // The common step (the next pair lies in the same query block) is a handful of scalar additions; what the step adds is
+    // kept in variables that turn to zero once every listed pair has been requested, so that the cursor then stays on the
+    // last pair without a test of its own.
+    int g_cur = -1, e_cur = -1, cnt_cur = 0, rem = 1, sub = 0;
+    int row_step = 2 * kSlab;
+    int64_t unit_step = 2 * kDsUnitBytes;                   // to the next pair inside a 128-row tile
+    int64_t tile_step = (int64_t)(nsub_k * 4 - 4) * kDsUnitBytes;  // on top of it, from a tile's last pair to the next tile's first
     ConstIdx idx_cur = nullptr;
-    int64_t row_next = 0, head_row0 = 0;
-    auto next_block = [&]() {  // position row_next on the first row of the next listed query block, if any
+    int64_t row_next = 0, head_row0 = 0, unit_next = 0, slot0_cur = 0;
+    auto enter_head = [&](int g) {  // list row, first query row and first pair number of query head g of the group
+      const int64_t lr = list_row(g);
+      cnt_cur = k_cnt[lr];
+      idx_cur = const_idx(p.k_idx + lr * row_len);
+      const int64_t bh = (int64_t)b * p.Hq + hkv * group + g;
+      head_row0 = bh * p.Sq;
+      if constexpr (kHandOver) {
+        const ConstIdx pb = const_idx(p.pair_base);
+        slot0_cur = pb[lr] + (p.mask_bh == 1 ? bh * pb[p.nK] : 0);
+      }
+    };
+    auto enter_block = [&](int first_sub) {  // entry e_cur of the current head, starting at slab first_sub (a multiple of 4)
+      row_next = head_row0 + (int64_t)idx_cur[e_cur] * p.q_block + first_sub * kSlab;
+      if constexpr (kHandOver)
+        unit_next = (slot0_cur + e_cur) * pair_bytes + ((int64_t)((first_sub >> 2) * nsub_k + t_key) * 4) * kDsUnitBytes;
+      sub = first_sub;
+      rem = (nsub - first_sub) >> 1;
+    };
+    auto next_block = [&]() {  // first pair of the next listed query block, if any
       ++e_cur;
-      while (e_cur >= cnt_cur) {
-        if (++g_cur >= group) { more = false; return; }
-        const int64_t lr = list_row(g_cur);
-        cnt_cur = k_cnt[lr];
-        idx_cur = const_idx(p.k_idx + lr * row_len);
-        head_row0 = ((int64_t)b * p.Hq + hkv * group + g_cur) * p.Sq;
+      while (e_cur >= cnt_cur && g_cur + 1 < group) {
+        enter_head(++g_cur);
         e_cur = 0;
       }
-      row_next = head_row0 + (kTiled ? (int64_t)(idx_cur[e_cur] >> 8) * kSlab : (int64_t)idx_cur[e_cur] * p.q_block);
-      rem = nsub;
+      if (e_cur < cnt_cur) {
+        enter_block(0);
+      } else {  // nothing left: every further step repeats the last pair
+        row_step = 0;
+        unit_step = 0;
+        tile_step = 0;
+        rem = 1 << 30;
+      }
     };
-    auto advance = [&]() {
-      if (!more) return;
-      if (--rem == 0) next_block(); else row_next += kSlab;
+    auto advance = [&]() {  // to the next pair
+      if (rem == 1) {
+        next_block();
+      } else {
+        --rem;
+        row_next += row_step;
+        sub += 2;
+        // units of a pair are ordered (128-row tile of the block, 32-key slab, slab inside the tile)
+        if constexpr (kHandOver) unit_next += unit_step + ((sub & 3) ? 0 : tile_step);
+      }
     };
     // Nine copies per wave request one slab (Q rows, dO rows, statistics), by the two waves of the slab's parity.  Every
     // step issues them, so that the count of copies in flight is the same at every wait; once the lists are exhausted
@@ -198,72 +239,22 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
       else if (i < 8) dma16(dst + kSlabBytes + dma_dst + (i - 4) * 4 * kRowBytes, dobase + row * kRowBytes, dma_off[i - 4]);
       else dma4(dst + 2 * kSlabBytes, stbase + row * 4, stat_off);
     };
-    // Slabs are numbered in list order; slabs 2i and 2i+1 form pair i, the first for the waves of parity 0, the second for
-    // those of parity 1.  A parity keeps three buffers: ring buffer 3 * par + (i % 3) holds its slab of pair i.
-    auto request_pair = [&](int buf) {
-      const int64_t r0 = row_next;
-      advance();
-      const int64_t r1 = row_next;
-      advance();
-      issue_copy(3 * par + buf, par ? r1 : r0);
-    };
+    // A parity keeps three buffers: ring buffer 3 * par + (i % 3) holds its slab of pair i.
     if (parts == 1) {
       next_block();
     } else {  // start in the middle of the lists
       g_cur = g_begin;
-      const int64_t lr = list_row(g_cur);
-      cnt_cur = k_cnt[lr];
-      idx_cur = const_idx(p.k_idx + lr * row_len);
-      head_row0 = ((int64_t)b * p.Hq + hkv * group + g_cur) * p.Sq;
+      enter_head(g_cur);
       e_cur = e_begin;
-      row_next = head_row0 + (int64_t)idx_cur[e_cur] * p.q_block + sub_begin * kSlab;
-      rem = nsub - sub_begin;
+      enter_block(sub_begin);
     }
-    request_pair(0);
-    request_pair(1);
-
-    // dS hand-over: (query head of the group, list entry, slab inside the query block) of the slab whose dS this wave forms
-    // next, and the pair number of entry 0 of that head's list row
-    int h_g = -1, h_e = -1, h_s = 0, h_cnt = 0;
-    int64_t h_slot0 = 0;
-    const int64_t pair_bytes = (int64_t)p.q_block * p.k_block * 2;
-    const int nsub_k = p.k_block / kSlab;
-    const int t_key = 4 * ((kt * TK - kblk * p.k_block) / TK) + 2 * kg;  // this wave's first 32-key slab inside the key block
-    const int ho_off0 = ds_unit_store_off(0, lane), ho_off1 = ds_unit_store_off(1, lane);
-    auto ho_next_entry = [&]() {
-      ++h_e;
-      while (h_e >= h_cnt) {
-        if (++h_g >= group) return;
-        const int64_t lr = list_row(h_g);
-        h_cnt = k_cnt[lr];
-        const ConstIdx pb = const_idx(p.pair_base);
-        const int64_t bh = (int64_t)b * p.Hq + hkv * group + h_g;
-        h_slot0 = pb[lr] + (p.mask_bh == 1 ? bh * pb[p.nK] : 0);
-        h_e = 0;
-      }
-    };
-    auto ho_advance = [&](int n) {
-      h_s += n;
-      if (h_s >= nsub) {  // nsub >= 4 > n
-        h_s -= nsub;
-        ho_next_entry();
-      }
-    };
-    if constexpr (kHandOver) {
-      if (parts == 1) {
-        ho_next_entry();
-      } else {
-        h_g = g_begin;
-        const int64_t lr = list_row(h_g);
-        h_cnt = k_cnt[lr];
-        const ConstIdx pb = const_idx(p.pair_base);
-        const int64_t bh = (int64_t)b * p.Hq + hkv * group + h_g;
-        h_slot0 = pb[lr] + (p.mask_bh == 1 ? bh * pb[p.nK] : 0);
-        h_e = e_begin;
-        h_s = sub_begin;
-      }
-      ho_advance(par);
-    }
+    // pairs 0 and 1 are requested here; their dS units wait in unit_cur (the slab whose softmax is next) and unit_nxt
+    int64_t unit_cur = unit_next + par * kDsUnitBytes;
+    issue_copy(3 * par + 0, row_next + par * kSlab);
+    advance();
+    int64_t unit_nxt = unit_next + par * kDsUnitBytes;
+    issue_copy(3 * par + 1, row_next + par * kSlab);
+    advance();
     wait_vmem<0>();
     __syncthreads();
 
@@ -415,47 +406,44 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
         for (int e = 0; e < 8; ++e) { pk[grp][j][e] = (__bf16)0.f; dsk[grp][j][e] = (__bf16)0.f; }
     scores(std::false_type{}, 0, 0, 0, nullptr);
     // Iteration t: slab t lives in buffer t % 3, slab t-1 in (t+2) % 3, slab t+1 in (t+1) % 3.  The first iteration adds
-    // nothing (P = dS = 0 against the finite rows of slab 0); the last one, t = nlocal, only adds slab nlocal-1 (its
-    // arithmetic runs on stale registers and is dropped), so that every wave passes the same barriers.
+    // nothing (P = dS = 0 against the finite rows of slab 0).  The loop body has no branch but the cursor's change of block;
+    // the wave's last slab is handled behind the loop.
     int cur = 0, prev = 0, nxt = kStageBytes;
-    bool stores_in_flight = false;  // did the previous iteration end with four dS stores?
-    for (int t = 0; t <= nlocal; ++t) {
+    for (int t = 0; t + 1 < nlocal; ++t) {
       softmax_and_accumulate(cur, prev);
-      char* ds_unit = nullptr;  // where dS_t goes (null: nothing to store)
-      if constexpr (kHandOver) {
-        if (t < nlocal)
-          ds_unit = reinterpret_cast<char*>(p.ds_ws) + (h_slot0 + h_e) * pair_bytes +
-                    ((int64_t)((h_s >> 2) * nsub_k + t_key) * 4 + (h_s & 3)) * kDsUnitBytes;
-        ho_advance(2);
-      }
+      char* ds_unit = nullptr;  // where dS_t goes
+      if constexpr (kHandOver) ds_unit = reinterpret_cast<char*>(p.ds_ws) + unit_cur;
+      // slab t+2 will replace slab t-1 (past the end of the lists: a repeat of the last slab that nobody reads); its copies
+      // are issued in between the matrix instructions of scores().  The cursor moves on here, while the last matrix
+      // instructions of this slab still run.
+      const int64_t req_row = row_next + par * kSlab;
+      unit_cur = unit_nxt;
+      unit_nxt = unit_next + par * kDsUnitBytes;
+      advance();
       // this wave's copies of slab t+1, requested during the previous iteration, must have landed; the four dS stores issued
-      // after them may still be on their way (the counter covers loads and stores alike, in issue order)
-      if (kHandOver && stores_in_flight) wait_vmem<4>(); else wait_vmem<0>();
+      // after them may still be on their way (the counter covers loads and stores alike, in issue order; before the first
+      // iteration nothing is in flight)
+      if constexpr (kHandOver) wait_vmem<4>(); else wait_vmem<0>();
       __syncthreads();  // everybody is done with slab t-1 and everybody's copies of slab t+1 have landed
       const int freed = nxt + kStageBytes == 3 * kStageBytes ? 0 : nxt + kStageBytes;  // buffer of slab t-1 = buffer of slab t+2
-      // slab t+2 replaces slab t-1 (past the end of the lists: a repeat of the last slab that nobody reads); its copies are
-      // issued in between the matrix instructions of scores()
-      const int64_t r0 = row_next;
-      advance();
-      const int64_t r1 = row_next;
-      advance();
       const uint32_t req_dst = ring_dst + 3 * par * kStageBytes + freed;
-      stores_in_flight = ds_unit != nullptr;
-      if (t + 1 < nlocal) {
-        scores(std::true_type{}, nxt, req_dst, par ? r1 : r0, ds_unit);
-      } else if constexpr (kHandOver) {
-        if (ds_unit != nullptr) {  // the wave's last slab: no scores() follows that could carry its stores
-#pragma unroll
-          for (int grp = 0; grp < 2; ++grp) {
-            __builtin_nontemporal_store(dsk[grp][0], reinterpret_cast<bf16x8*>(ds_unit + grp * 4 * kDsUnitBytes + ho_off0));
-            __builtin_nontemporal_store(dsk[grp][1], reinterpret_cast<bf16x8*>(ds_unit + grp * 4 * kDsUnitBytes + ho_off1));
-          }
-        }
-      }
+      scores(std::true_type{}, nxt, req_dst, req_row, ds_unit);
       prev = cur;
       cur = nxt;
       nxt = freed;
     }
+    // the wave's last slab: no scores() follows that could carry its dS stores
+    softmax_and_accumulate(cur, prev);
+    if constexpr (kHandOver) {
+      char* ds_unit = reinterpret_cast<char*>(p.ds_ws) + unit_cur;
+#pragma unroll
+      for (int grp = 0; grp < 2; ++grp) {
+        __builtin_nontemporal_store(dsk[grp][0], reinterpret_cast<bf16x8*>(ds_unit + grp * 4 * kDsUnitBytes + ho_off0));
+        __builtin_nontemporal_store(dsk[grp][1], reinterpret_cast<bf16x8*>(ds_unit + grp * 4 * kDsUnitBytes + ho_off1));
+      }
+    }
+    // ... and its share of dV, dK (the arithmetic of this call runs on stale registers and is dropped)
+    softmax_and_accumulate(nxt, cur);
     wait_vmem<0>();
     __syncthreads();  // no copy is writing LDS any more; V and the ring are free
 
