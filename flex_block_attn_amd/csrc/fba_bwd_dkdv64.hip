@@ -258,20 +258,20 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     wait_vmem<0>();
     __syncthreads();
 
-    // per-lane fetch addresses with the wave's share folded in: slab addresses carry the parity's three buffers, V
-    // addresses the wave's 64 keys; what remains (buffer, Q or dO, key group, row group) is a compile-time displacement
+    // Per-lane fetch addresses with the wave's share folded in: slab addresses carry the parity's three buffers, V
+    // addresses the wave's 64 keys.  One register each: the operand step (row-major fetches) and the column block and row
+    // half (transposed fetches) only move the 16-byte chunk inside a 256-byte row, chunk c of row r living in slot
+    // c ^ swz(r), so they are exclusive-ors with constants below 256; everything added here is a multiple of 256.
+    static_assert(kStageBytes % 256 == 0 && kTileBase % 256 == 0 && kSlabBytes % 256 == 0, "the exclusive-ors below touch bits 5..7");
     const LdsPtr lds = lds_ptr(smem);
-    LdsPtr q_ptr[8], v_ptr[8], t_ptr[4][2];
-#pragma unroll
-    for (int ks = 0; ks < 8; ++ks) {
-      q_ptr[ks] = lds + rm.rd[ks] + par * 3 * kStageBytes;
-      v_ptr[ks] = lds + rm.rd[ks] + kTileBase + kg * 2 * kSlabBytes;
-    }
-#pragma unroll
-    for (int mb = 0; mb < 4; ++mb) {
-      t_ptr[mb][0] = lds + tr.rd[mb][0] + par * 3 * kStageBytes;
-      t_ptr[mb][1] = lds + tr.rd[mb][1] + par * 3 * kStageBytes;
-    }
+    const LdsPtr q_base = lds + rm.rd[0] + par * 3 * kStageBytes;
+    const LdsPtr v_base = lds + rm.rd[0] + kTileBase + kg * 2 * kSlabBytes;
+    const LdsPtr t_base = lds + tr.rd[0][0] + par * 3 * kStageBytes;
+    auto flip = [](LdsPtr ptr, uint32_t bits) { return (LdsPtr)(uintptr_t)((uint32_t)(uintptr_t)ptr ^ bits); };
+    auto row_major = [&](LdsPtr base, int ks) { return flip(base, 32u * ks); };  // operand step ks of a slab (base: step 0)
+    auto transposed = [&](LdsPtr base, int mb, int half) {                        // column block mb, rows +8 * half
+      return flip(base, (uint32_t)(mb << 6 | half << 5)) + half * 8 * kRowBytes;
+    };
     const LdsPtr st_ptr = lds + par * 3 * kStageBytes + 2 * kSlabBytes + 16 * h;
 #pragma unroll
     for (int grp = 0; grp < 2; ++grp)
@@ -286,8 +286,12 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     bf16x8 pk[2][2], dsk[2][2];  // P and dS of the previous slab, packed as B operands
 
     // S, dP of the slab in the buffer at byte offset `so` against this wave's 64 keys: every Q / dO operand feeds both key
-    // groups.  The operands of step ks+1 are requested before the matrix instructions of step ks are issued; the scheduling
-    // fences keep the compiler from moving them back next to their use, where the wave would wait for every fetch.
+    // groups.  S comes first, so that while the matrix pipe works on dP the vector unit can already turn S of the first key
+    // group into P = exp2(S c - lse) (in place): a wave alone on its SIMD pays for every instruction it issues, and the
+    // other phase, softmax_and_accumulate(), has more arithmetic than its matrix instructions cover, this one less.
+    // Matrix instructions go in fours, two operand steps each; the operands of the next four are requested before a four
+    // is issued, and the scheduling fences keep the compiler from moving the requests back next to their use, where the
+    // wave would wait for every fetch.
     auto scores = [&](auto extras_c, int so, uint32_t req_dst, int64_t req_row, char* ds_unit) {
       constexpr bool kExtras = decltype(extras_c)::value;  // false for the wave's first slab: nothing to copy or store yet
       // accumulator element 4g + e of half-wave h is query row 8g + 4h + e of the slab; dP starts from -delta of its row
@@ -300,40 +304,75 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
           dp[0][4 * g + e] = d4[e]; dp[1][4 * g + e] = d4[e];
         }
       }
-      bf16x8 qf = lds_read_b128(q_ptr[0] + so), dof = lds_read_b128(q_ptr[0] + so + kSlabBytes);
-      bf16x8 vf0 = lds_read_b128(v_ptr[0]), vf1 = lds_read_b128(v_ptr[0] + kSlabBytes);
+      LdsPtr qs = q_base + so, vs = v_base;
+      asm volatile("" : "+v"(qs), "+v"(vs));  // one register each; the eight addresses are formed where they are used
+      bf16x8 qa = lds_read_b128(row_major(qs, 0)), qb = lds_read_b128(row_major(qs, 1));
+      bf16x8 da, db, va0, va1, vb0, vb1;
+      f32x4 l4;  // lse * log2(e) of the rows whose P comes next
 #pragma unroll
-      for (int ks = 0; ks < 8; ++ks) {
-        bf16x8 qf_n = qf, dof_n = dof, vf0_n = vf0, vf1_n = vf1;
-        if (ks < 7) {
-          qf_n = lds_read_b128(q_ptr[ks + 1] + so);
-          dof_n = lds_read_b128(q_ptr[ks + 1] + so + kSlabBytes);
-          vf0_n = lds_read_b128(v_ptr[ks + 1]);
-          vf1_n = lds_read_b128(v_ptr[ks + 1] + kSlabBytes);
+      for (int j = 0; j < 4; ++j) {  // S: operand steps 2j, 2j+1
+        bf16x8 qa_n = qa, qb_n = qb;
+        if (j < 3) {
+          qa_n = lds_read_b128(row_major(qs, 2 * j + 2));
+          qb_n = lds_read_b128(row_major(qs, 2 * j + 3));
+        } else {  // the first operands of dP
+          da = lds_read_b128(row_major(qs, 0) + kSlabBytes);
+          va0 = lds_read_b128(row_major(vs, 0));
+          va1 = lds_read_b128(row_major(vs, 0) + kSlabBytes);
+          db = lds_read_b128(row_major(qs, 1) + kSlabBytes);
+          vb0 = lds_read_b128(row_major(vs, 1));
+          vb1 = lds_read_b128(row_major(vs, 1) + kSlabBytes);
+          l4 = lds_read_f32x4(st_ptr + so);
         }
         __builtin_amdgcn_sched_barrier(0);
-        s[0] = mfma32(qf, kreg[0][ks], s[0]);
-        s[1] = mfma32(qf, kreg[1][ks], s[1]);
-        // the copies of the slab after next and the dS stores of the slab before are issued one at a time between the
-        // matrix instructions: a wave alone on its SIMD pays for every cycle a memory instruction takes to issue
-        // (copies first, stores last: the wait before the next barrier then lets the four youngest operations, the stores,
-        // stay in flight)
+        // the copies of the slab after next are issued one at a time between the matrix instructions (copies first, the dS
+        // stores of the slab before last: the wait before the next barrier then lets the four youngest operations, the
+        // stores, stay in flight)
+        s[0] = mfma32(qa, kreg[0][2 * j], s[0]);
         if constexpr (kExtras) {
-          if (ks < 4) issue_copy_part(2 * ks, req_dst, req_row);
+          if (j < 3) issue_copy_part(3 * j, req_dst, req_row);
         }
-        dp[0] = mfma32(dof, vf0, dp[0]);
+        s[1] = mfma32(qa, kreg[1][2 * j], s[1]);
         if constexpr (kExtras) {
-          if (ks < 4) issue_copy_part(2 * ks + 1, req_dst, req_row);
-          else if (ks == 4) issue_copy_part(8, req_dst, req_row);
+          if (j < 3) issue_copy_part(3 * j + 1, req_dst, req_row);
         }
-        dp[1] = mfma32(dof, vf1, dp[1]);
-        if constexpr (kHandOver && kExtras) {
-          if (ks >= 4)  // scores() runs only while the wave has a further slab, so slab t exists and ds_unit is set
-            __builtin_nontemporal_store(dsk[(ks >> 1) & 1][ks & 1],
-                                        reinterpret_cast<bf16x8*>(ds_unit + ((ks >> 1) & 1) * 4 * kDsUnitBytes + ((ks & 1) ? ho_off1 : ho_off0)));
+        s[0] = mfma32(qb, kreg[0][2 * j + 1], s[0]);
+        if constexpr (kExtras) {
+          if (j < 3) issue_copy_part(3 * j + 2, req_dst, req_row);
+        }
+        s[1] = mfma32(qb, kreg[1][2 * j + 1], s[1]);
+        __builtin_amdgcn_sched_barrier(0);
+        qa = qa_n; qb = qb_n;
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {  // dP: operand steps 2j, 2j+1; P of the first key group, rows 8j + 4h + 0..3
+        bf16x8 da_n = da, db_n = db, va0_n = va0, va1_n = va1, vb0_n = vb0, vb1_n = vb1;
+        f32x4 l4_n = l4;
+        if (j < 3) {
+          da_n = lds_read_b128(row_major(qs, 2 * j + 2) + kSlabBytes);
+          va0_n = lds_read_b128(row_major(vs, 2 * j + 2));
+          va1_n = lds_read_b128(row_major(vs, 2 * j + 2) + kSlabBytes);
+          db_n = lds_read_b128(row_major(qs, 2 * j + 3) + kSlabBytes);
+          vb0_n = lds_read_b128(row_major(vs, 2 * j + 3));
+          vb1_n = lds_read_b128(row_major(vs, 2 * j + 3) + kSlabBytes);
+          l4_n = lds_read_f32x4(st_ptr + so + 32 * (j + 1));
         }
         __builtin_amdgcn_sched_barrier(0);
-        qf = qf_n; dof = dof_n; vf0 = vf0_n; vf1 = vf1_n;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (e == 0) dp[0] = mfma32(da, va0, dp[0]);
+          if (e == 1) dp[1] = mfma32(da, va1, dp[1]);
+          if (e == 2) dp[0] = mfma32(db, vb0, dp[0]);
+          if (e == 3) dp[1] = mfma32(db, vb1, dp[1]);
+          float pv = fast_exp2(__builtin_fmaf(s[0][4 * j + e], c, -l4[e]));
+          asm volatile("" : "+v"(pv));  // keeps this element's arithmetic behind its matrix instruction
+          s[0][4 * j + e] = pv;
+        }
+        if constexpr (kHandOver && kExtras) {  // scores() runs only while the wave has a further slab, so ds_unit is set
+          __builtin_nontemporal_store(dsk[j >> 1][j & 1], reinterpret_cast<bf16x8*>(ds_unit + (j >> 1) * 4 * kDsUnitBytes + ((j & 1) ? ho_off1 : ho_off0)));
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        da = da_n; db = db_n; va0 = va0_n; va1 = va1_n; vb0 = vb0_n; vb1 = vb1_n; l4 = l4_n;
       }
     };
 
@@ -343,16 +382,18 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     // accumulator elements of arithmetic; the operands and statistics of group n+1 are requested before group n starts.
     auto softmax_and_accumulate = [&](int so, int po) {
       bf16x2 pw[2][8], dw[2][8];  // new P and dS, packed: [key group][register pair]
+      LdsPtr ts = t_base + po;
+      asm volatile("" : "+v"(ts));
       auto fetch_dv = [&](int n) {
-        const int roff = po + 16 * (n >> 2) * kRowBytes, mb = n & 3;
-        return cat(lds_read_tr(t_ptr[mb][0] + kSlabBytes + roff), lds_read_tr(t_ptr[mb][1] + kSlabBytes + roff));
+        const int roff = 16 * (n >> 2) * kRowBytes, mb = n & 3;
+        return cat(lds_read_tr(transposed(ts, mb, 0) + kSlabBytes + roff), lds_read_tr(transposed(ts, mb, 1) + kSlabBytes + roff));
       };
       auto fetch_dk = [&](int n) {
-        const int roff = po + 16 * (n >> 2) * kRowBytes, mb = n & 3;
-        return cat(lds_read_tr(t_ptr[mb][0] + roff), lds_read_tr(t_ptr[mb][1] + roff));
+        const int roff = 16 * (n >> 2) * kRowBytes, mb = n & 3;
+        return cat(lds_read_tr(transposed(ts, mb, 0) + roff), lds_read_tr(transposed(ts, mb, 1) + roff));
       };
       bf16x8 adv = fetch_dv(0), adk = fetch_dk(0);
-      f32x4 l4 = lds_read_f32x4(st_ptr + so);
+      f32x4 l4 = {0.f, 0.f, 0.f, 0.f};  // statistics of the second key group's rows only: scores() left P of the first group
 #pragma unroll
       for (int n = 0; n < 8; ++n) {  // n = 4 j + mb for the matrix work, 4 grp + g for the arithmetic
         bf16x8 adv_n = adv, adk_n = adk;
@@ -360,7 +401,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
         if (n < 7) {
           adv_n = fetch_dv(n + 1);
           adk_n = fetch_dk(n + 1);
-          l4_n = lds_read_f32x4(st_ptr + so + 32 * ((n + 1) & 3));
+          if (n >= 3) l4_n = lds_read_f32x4(st_ptr + so + 32 * ((n + 1) & 3));
         }
         __builtin_amdgcn_sched_barrier(0);
         const int j = n >> 2, mb = n & 3, grp = n >> 2, g = n & 3;
@@ -371,7 +412,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
           if (e == 1) mfma32_acc(acc_v[1][mb], adv, pk[1][j]);
           if (e == 2) mfma32_acc(acc_k[0][mb], adk, dsk[0][j]);
           if (e == 3) mfma32_acc(acc_k[1][mb], adk, dsk[1][j]);
-          pv[e] = fast_exp2(__builtin_fmaf(s[grp][4 * g + e], c, -l4[e]));
+          pv[e] = grp == 0 ? s[0][4 * g + e] : fast_exp2(__builtin_fmaf(s[1][4 * g + e], c, -l4[e]));
           dsv[e] = pv[e] * dp[grp][4 * g + e];
           if (e & 1) {
             bf16x2 p2 = __builtin_convertvector((f32x2){pv[e - 1], pv[e]}, bf16x2);
