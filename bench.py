@@ -157,6 +157,18 @@ def sustained_mfma_tflops(dev, data):
     return wgs * 4.0 * iters * 4 * 32768 / (ms * 1e-3) * 1e-12
 
 
+def streaming_read_gbs(dev):
+    """GB/s at which a kernel that only reads (fba_probe_read: streaming 16-byte loads, nothing stored) pulls 4 GiB from device memory."""
+    from flex_block_attn_amd import _lib
+    from flex_block_attn_amd.interface import _ptr, _stream
+
+    nbytes = 4 << 30
+    src = torch.empty((nbytes,), dtype=torch.uint8, device=dev).fill_(1)
+    sink = torch.zeros((1,), dtype=torch.int32, device=dev)
+    ms = statistics.median(time_events(lambda: _lib.call("fba_probe_read", _ptr(src), nbytes, _ptr(sink), 2048, _stream()), 1, 5))
+    return nbytes / (ms * 1e-3) * 1e-9
+
+
 def probe_atomics():
     """fp32 atomic adds of 512-byte rows (one query row of dQ) at random rows of a [24 * 30720, 128] fp32 buffer, through
     torch's index_add_ (a gather of src rows + one hardware atomic add per element), against a plain copy of the same bytes.
@@ -319,6 +331,12 @@ def main():
     if roofline["bound"] == "mfma":
         roofline["sustained_peak"] = sustained["normal"]
         roofline["frac_of_sustained"] = roofline["achieved"] / sustained["normal"]
+    # ... and what a kernel that only reads pulls from device memory: the yardstick of the kernel that reads dS back
+    read_gbs = streaming_read_gbs(dev)
+    log(f"read-only streaming kernel: {read_gbs:.0f} GB/s (nominal peak {PEAK_HBM_GBS:.0f})")
+    if hand_over:
+        rooflines["bwd_dq_from_ds"]["streaming_read_GB/s"] = read_gbs
+        rooflines["bwd_dq_from_ds"]["frac_of_streaming_read"] = rooflines["bwd_dq_from_ds"]["achieved"] / read_gbs
 
     mask_bytes = mask.numel() + 4 * (2 * nnz // (1 if mask.dim() == 4 else B * H) + lists.mask_bh * (lists.nQ + lists.nK))
     compaction = {"ms": kms["mask_compact"]["mean_ms"], "algorithmic_bytes": mask_bytes, "GB/s": mask_bytes / (kms["mask_compact"]["mean_ms"] * 1e-3) * 1e-9, "peak_GB/s": PEAK_HBM_GBS}
@@ -335,6 +353,7 @@ def main():
         "kernels_ms": {n: kms[n]["mean_ms"] for n in kms},
         "rooflines": rooflines,
         "bare_mfma_loop_TFLOP/s": sustained,
+        "streaming_read_GB/s": read_gbs,
         "mask_compaction": compaction,
     }
     if mask_fn:

@@ -27,6 +27,7 @@ SIGNATURES = {
     "fba_fwd": (_c_i32, [_c_ptr] * 7 + [_c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
     "fba_bwd": (_c_i32, [_c_ptr] * 14 + [_c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
     "fba_probe_mfma": (_c_i32, [_c_ptr, _c_ptr, _c_i32, _c_i32, _c_ptr]),
+    "fba_probe_read": (_c_i32, [_c_ptr, _c_i64, _c_ptr, _c_i32, _c_ptr]),
     "fba_pair_slots": (_c_i32, [_c_ptr] * 4 + [_c_i64, _c_i32, _c_i32, _c_ptr, _c_ptr, _c_ptr]),
     "fba_bwd_handover": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_ptr] * 9 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
     "fba_bwd_dkdv_handover": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_ptr] * 3 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),

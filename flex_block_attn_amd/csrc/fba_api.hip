@@ -79,7 +79,7 @@ int check_split_ws(const void* ws, int64_t bytes) {
 
 extern "C" {
 
-int32_t fba_version(void) { return 2000; }
+int32_t fba_version(void) { return 2001; }
 
 const char* fba_last_error(void) { return g_err; }
 
@@ -319,6 +319,14 @@ int32_t fba_probe_mfma(const float* src, float* sink, int32_t work_groups, int32
   if (work_groups <= 0 || iters <= 0) return fail(FBA_ERR_INVALID, "work_groups and iters must be positive (got %d %d)", work_groups, iters);
   if (!sink) return fail(FBA_ERR_INVALID, "sink is null");
   hipError_t e = fba::launch_probe_mfma(src, sink, work_groups, iters, (hipStream_t)hip_stream);
+  return e == hipSuccess ? FBA_OK : hip_fail(e, "probe launch");
+}
+
+int32_t fba_probe_read(const void* src, int64_t bytes, uint32_t* sink, int32_t work_groups, void* hip_stream) {
+  if (work_groups <= 0 || bytes <= 0 || bytes % 32768 != 0)
+    return fail(FBA_ERR_INVALID, "work_groups must be positive and bytes a positive multiple of 32768 (got %d %lld)", work_groups, (long long)bytes);
+  if (!src || !sink) return fail(FBA_ERR_INVALID, "src or sink is null");
+  hipError_t e = fba::launch_probe_read(src, bytes, sink, work_groups, (hipStream_t)hip_stream);
   return e == hipSuccess ? FBA_OK : hip_fail(e, "probe launch");
 }
 

@@ -124,6 +124,7 @@ hipError_t launch_bwd_dq_from_ds(BwdParams p, hipStream_t stream);
 hipError_t launch_partial_sum(const float* ws, int parts, int64_t slot_floats, __bf16* out, int64_t out_row0, int n_items, float scale,
                               hipStream_t stream);
 hipError_t launch_probe_mfma(const float* src, float* sink, int work_groups, int iters, hipStream_t stream);
+hipError_t launch_probe_read(const void* src, int64_t bytes, uint32_t* sink, int work_groups, hipStream_t stream);
 hipError_t launch_pair_slots(const int32_t* q_cnt, const int32_t* q_idx, const int32_t* k_cnt, const int32_t* k_idx, int64_t mask_bh,
                              int nQ, int nK, int32_t* pair_base, int32_t* q_slot, hipStream_t stream);
 hipError_t launch_tile_slots(const int32_t* kt_cnt, const int32_t* kt_ent, int64_t mask_bh, int n_qt, int n_kt, int n_qs,

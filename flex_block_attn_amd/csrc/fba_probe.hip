@@ -8,6 +8,8 @@
 
 namespace fba {
 
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
 __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void probe_mfma_kernel(const float* __restrict__ src,
                                                                                          float* __restrict__ sink, int iters) {
   bf16x8 a, b;
@@ -29,6 +31,29 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void probe_mfm
 #pragma unroll
   for (int r = 0; r < 16; ++r) s += c0[r] + c1[r] + c2[r] + c3[r];
   sink[(size_t)blockIdx.x * 256 + threadIdx.x] = s;
+}
+
+// Diagnostic: what a kernel that only reads can pull from device memory.  Every lane keeps eight 16-byte loads with the
+// streaming hint in flight and folds them into one word; `sink` is written only if that word has an unlikely value, so
+// the loop cannot be dropped.  The caller times the launch over a buffer much larger than the caches.
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void probe_read_kernel(const u32x4* __restrict__ src, int64_t n_vec,
+                                                                                         uint32_t* __restrict__ sink) {
+  constexpr int kInFlight = 8;
+  u32x4 acc = {0, 0, 0, 0};
+  const int64_t stride = (int64_t)gridDim.x * 256 * kInFlight;
+  for (int64_t i = (int64_t)blockIdx.x * 256 * kInFlight + threadIdx.x; i + 256 * (kInFlight - 1) < n_vec; i += stride) {
+    u32x4 v[kInFlight];
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) v[u] = __builtin_nontemporal_load(src + i + 256 * u);
+#pragma unroll
+    for (int u = 0; u < kInFlight; ++u) acc ^= v[u];
+  }
+  if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x5eed1e55u) sink[0] = 1;
+}
+
+hipError_t launch_probe_read(const void* src, int64_t bytes, uint32_t* sink, int work_groups, hipStream_t stream) {
+  hipLaunchKernelGGL(probe_read_kernel, dim3(work_groups), dim3(256), 0, stream, reinterpret_cast<const u32x4*>(src), bytes / 16, sink);
+  return hipGetLastError();
 }
 
 hipError_t launch_probe_mfma(const float* src, float* sink, int work_groups, int iters, hipStream_t stream) {

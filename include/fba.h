@@ -233,6 +233,15 @@ int32_t fba_tile_permute(const void* x, void* out, int64_t n_seq, int32_t T, int
  */
 int32_t fba_probe_mfma(const float* src, float* sink, int32_t work_groups, int32_t iters, void* hip_stream);
 
+/*
+ * Diagnostic, no counterpart in the reference: `work_groups` x 256 lanes read the `bytes` at src (device memory, a
+ * multiple of 32 KiB) once, eight 16-byte streaming loads per lane in flight, and write nothing (sink: 4 bytes of device
+ * memory that stay as they are unless the data folds to one particular word).  Timed by the caller over a buffer much
+ * larger than the caches it gives the rate at which a read-only kernel pulls from device memory on this GPU, the
+ * yardstick for the kernel that reads the dS workspace back.
+ */
+int32_t fba_probe_read(const void* src, int64_t bytes, uint32_t* sink, int32_t work_groups, void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -683,6 +683,23 @@ def test_matrix_pipe_probe(gpu):
     assert torch.equal(sink, torch.full_like(sink, 4.0 * 10 * 64))
 
 
+def test_read_probe_reads_and_leaves_its_sink(gpu):
+    """fba_probe_read: reads the buffer and stores nothing: the sink keeps its value, except for data that folds to the
+    one word the kernel tests for (a buffer holding that word once and zeros elsewhere)."""
+    from flex_block_attn_amd import _lib
+    from flex_block_attn_amd.interface import _ptr, _stream
+
+    src = torch.randint(0, 2 ** 31 - 1, (32768 * 4 // 4,), dtype=torch.int32, device=gpu)
+    sink = torch.full((1,), 7, dtype=torch.int32, device=gpu)
+    _lib.call("fba_probe_read", _ptr(src), src.numel() * 4, _ptr(sink), 3, _stream())
+    assert int(sink[0]) == 7
+    src.zero_()
+    src[12345] = 0x5EED1E55
+    _lib.call("fba_probe_read", _ptr(src), src.numel() * 4, _ptr(sink), 3, _stream())
+    torch.cuda.synchronize()
+    assert int(sink[0]) == 1  # the word was read by the lane that owns it
+
+
 @pytest.mark.parametrize("block_size", [64, 128, 384])
 def test_readme_usage_verbatim(oracle, gpu, block_size):
     """The reference README's usage section (README.md:24-53), run as written: its two imports, a list-of-lists

@@ -99,6 +99,8 @@ def test_c_abi_argument_validation(lib):
     assert h.fba_tile_permute(f, _fake(0x2000), 1, 6, 8, 9, 6, 8, 8, 128, 1, _null()) == lib.FBA_ERR_INVALID and b"divide" in h.fba_last_error()
     assert h.fba_tile_permute(f, f, 1, 6, 8, 8, 6, 8, 8, 128, 1, _null()) == lib.FBA_ERR_INVALID and b"alias" in h.fba_last_error()
     assert h.fba_probe_mfma(_null(), f, 0, 10, _null()) == lib.FBA_ERR_INVALID and h.fba_probe_mfma(_null(), _null(), 4, 10, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_probe_read(f, 32768 + 16, f, 4, _null()) == lib.FBA_ERR_INVALID and h.fba_probe_read(_null(), 32768, f, 4, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_probe_read(f, 32768, f, 0, _null()) == lib.FBA_ERR_INVALID
     # FbaError carries the code and the library's message
     with pytest.raises(lib.FbaError) as ei:
         lib.call("fba_mask_compact", f, 0, 4, 4, f, f, f, f, _null())
