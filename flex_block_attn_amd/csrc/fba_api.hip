@@ -54,10 +54,10 @@ int check_ptrs(std::initializer_list<std::pair<const char*, const void*>> ps) {
   return FBA_OK;
 }
 
-// Which dK/dV kernel runs on block lists: the one with 64 keys per wave (one wave per SIMD) by default.  It is 7-16 %
-// faster than the one with 32 keys per wave (two waves per SIMD) without the dS hand-over and 2-10 % faster with it
-// (a wave alone on its SIMD pays for every cycle its dS stores take to issue, which eats most of the gain).  Both do the
-// same arithmetic in the same order.  FBA_DKDV_KEYS_PER_WAVE = 32 or 64 overrides the choice (measurement of the two).
+// Which dK/dV kernel runs on block lists: the one with 64 keys per wave (one wave per SIMD) by default.  It is about 9 %
+// faster than the one with 32 keys per wave (two waves per SIMD) without the dS hand-over and about 7 % faster with it
+// (a wave alone on its SIMD pays for every cycle its dS stores take to issue).  Both do the same arithmetic in the same
+// order.  FBA_DKDV_KEYS_PER_WAVE = 32 or 64 overrides the choice (measurement of the two).
 hipError_t launch_dkdv_variant(fba::BwdParams& p, hipStream_t stream) {
   const char* env = getenv("FBA_DKDV_KEYS_PER_WAVE");
   const int keys = env ? atoi(env) : 64;
