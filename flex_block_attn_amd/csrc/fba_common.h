@@ -250,6 +250,11 @@ struct SlabDmaShared {
       if (has_v) dma16(slab_lds + dst[1], src, off[1]);
     }
   }
+  // Piece i (0 or 1) of the wave's share of a slab copy with four waves, for callers that spread the pieces out.
+  FBA_DEVICE void copy_piece(int i, uint32_t slab_lds, const char* src) const {
+    static_assert(kWaves == 4, "pieces exist with four waves only");
+    dma16(slab_lds + dst[i], src, off[i]);
+  }
   // Wait until only the copies this wave issued during the last two steps (one K and one V request each) may be in flight.
   FBA_DEVICE void wait_two_steps() const {
     if constexpr (kWaves == 4) {

@@ -55,8 +55,10 @@ FBA_DEVICE f32x16 qk_half(const FwdState& st, const char* k_half) {
   return s;
 }
 
-// O^T += V^T P^T for 32 keys: 8 MFMAs; consecutive MFMAs go to different accumulators.
-FBA_DEVICE void pv_half(FwdState& st, const char* v_half, const bf16x8 (&pk)[2]) {
+// O^T += V^T P^T for 32 keys: 8 MFMAs; consecutive MFMAs go to different accumulators.  `between(i)` runs behind matrix
+// instruction i: the place for the global -> LDS copies a step owes, which take a wave tens of cycles each to issue.
+template <typename Between>
+FBA_DEVICE void pv_half(FwdState& st, const char* v_half, const bf16x8 (&pk)[2], Between between) {
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
 #pragma unroll
@@ -64,8 +66,12 @@ FBA_DEVICE void pv_half(FwdState& st, const char* v_half, const bf16x8 (&pk)[2])
       const int roff = 16 * j * kRowBytes;
       const bf16x8 a = cat(lds_read_tr(v_half, st.tr.rd[mb][0] + roff), lds_read_tr(v_half, st.tr.rd[mb][1] + roff));
       st.acc_o[mb] = mfma32(a, pk[j], st.acc_o[mb]);
+      between(4 * j + mb);
     }
   }
+}
+FBA_DEVICE void pv_half(FwdState& st, const char* v_half, const bf16x8 (&pk)[2]) {
+  pv_half(st, v_half, pk, [](int) {});
 }
 
 // Raise the softmax reference if some row of the wave would otherwise see exponents above kLazy.  Until then
@@ -239,6 +245,16 @@ __global__ __attribute__((amdgpu_flat_work_group_size(64 * kWaves, 64 * kWaves),
     // (wave-uniform branches); rows switched off inside an active wave are dealt with by selects.
     const int wave_bits = 3 << (2 * wave);
     bool w_prev = false;  // did this wave form P for the previous slab?
+    // The copies a step requests (K_{t+5} into the buffer of K_{t+1}, V_{t+3} into that of V_{t-1}, both free behind the
+    // step's barrier) are issued by the following step, in between its first matrix instructions where the work-group
+    // has block lists and four waves: a copy takes a wave tens of cycles to issue, which the matrix pipe then covers.
+    // Every step requests both, so that the counter of copies in flight means the same thing at every wait; past the end
+    // of the list they repeat a listed slab into a buffer that nobody reads any more.
+    uint32_t owed_k_dst = 0, owed_v_dst = 0;
+    const char* owed_k_src = kp;
+    const char* owed_v_src = vp;
+    bool owed = false;
+    constexpr bool kSpread = !kTiled && kWaves == 4;
 
     // step t (t % 4 == R): O += P_{t-1} V_{t-1} | softmax(S_t) | S_{t+1} = K_{t+1} Q^T
     auto step = [&](auto ring_c, auto first_c, int t) {
@@ -247,8 +263,21 @@ __global__ __attribute__((amdgpu_flat_work_group_size(64 * kWaves, 64 * kWaves),
       const bool w_cur = !kTiled || (bits_cmp & wave_bits) != 0;
       const bool w_nxt = !kTiled || ((rem_cmp > 1 ? bits_cmp : bits_ahead) & wave_bits) != 0;
       // P_{t-1} was formed against the reference m of step t-1, so it must reach O before step t may raise m
-      if constexpr (!kFirst) {
-        if (w_prev) pv_half(st, v_lds + ((R + 3) & 3) * kSlabBytes, p_prev);
+      if constexpr (kSpread && !kFirst) {
+        pv_half(st, v_lds + ((R + 3) & 3) * kSlabBytes, p_prev, [&](int i) {
+          if (i == 0) dma.copy_piece(0, owed_k_dst, owed_k_src);
+          if (i == 2) dma.copy_piece(1, owed_k_dst, owed_k_src);
+          if (i == 4) dma.copy_piece(0, owed_v_dst, owed_v_src);
+          if (i == 6) dma.copy_piece(1, owed_v_dst, owed_v_src);
+        });
+      } else {
+        if (owed) {
+          copy_k(owed_k_dst, owed_k_src);
+          copy_v(owed_v_dst, owed_v_src);
+        }
+        if constexpr (!kFirst) {
+          if (w_prev) pv_half(st, v_lds + ((R + 3) & 3) * kSlabBytes, p_prev);
+        }
       }
       const bool active = !kTiled || (bits_cmp & group_bit) != 0;
       if (w_cur) softmax_reference(st, s_cur, active);
@@ -270,16 +299,16 @@ __global__ __attribute__((amdgpu_flat_work_group_size(64 * kWaves, 64 * kWaves),
       pin(p_prev[0]);
       pin(p_prev[1]);
       s_cur = s_nxt;
-      // K_{t+2} and V_t must have landed; the copies this wave requested after steps t-2 and t-1 may still fly
-      if (t + 5 < nsteps) dma.wait_two_steps(); else wait_vmem<0>();
+      // K_{t+2} and V_t must have landed; the copies requested by steps t-2 and t-1 may still fly
+      dma.wait_two_steps();
       __syncthreads();
-      const int64_t v_off = hist1;
+      owed_v_src = vp + hist1;
+      owed_v_dst = v_dst + ((R + 3) & 3) * kSlabBytes;
       hist1 = hist0;
-      if (t + 5 < nsteps) {
-        hist0 = next_off();
-        copy_k(k_dst + ((R + 1) & 3) * kSlabBytes, kp + hist0);
-      }
-      if (t + 3 < nsteps) copy_v(v_dst + ((R + 3) & 3) * kSlabBytes, vp + v_off);
+      hist0 = next_off();
+      owed_k_src = kp + hist0;
+      owed_k_dst = k_dst + ((R + 1) & 3) * kSlabBytes;
+      owed = true;
     };
     step(IC<0>{}, std::true_type{}, 0);
     step(IC<1>{}, std::false_type{}, 1);
@@ -292,6 +321,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(64 * kWaves, 64 * kWaves),
     }
     // O += P_{n-1} V_{n-1}
     if (w_prev) pv_half(st, v_lds + ((nsteps - 1) & 3) * kSlabBytes, p_prev);
+    wait_vmem<0>();  // no copy may still be writing LDS when the work-group gives it back
   }
 
   const float l = sum_halves(st.l_run);
