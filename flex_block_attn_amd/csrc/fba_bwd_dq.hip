@@ -105,9 +105,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   int e_next = e_begin + 1, rem = nsub - sub_begin;
   int64_t src_off = nsteps > 0 ? key_block(e_begin) * block_bytes + (int64_t)sub_begin * kSlabBytes : 0;
   int blk_next = e_next < cnt ? key_block(e_next) : 0;
-  auto copy_next = [&](int ring) {
-    dma.copy(ring_dst + ring * kPairBytes, kp + src_off);
-    dma.copy(ring_dst + ring * kPairBytes + kSlabBytes, vp + src_off);
+  auto next_off = [&]() -> int64_t {  // past the end of the list: offsets of some listed slab
+    const int64_t off = src_off;
     if (--rem == 0) {
       rem = nsub;
       src_off = blk_next * block_bytes;
@@ -116,16 +115,24 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     } else {
       src_off += kSlabBytes;
     }
+    return off;
+  };
+  auto copy_next = [&](int ring) {
+    const int64_t off = next_off();
+    dma.copy(ring_dst + ring * kPairBytes, kp + off);
+    dma.copy(ring_dst + ring * kPairBytes + kSlabBytes, vp + off);
   };
 
-  // S^T and dP^T of one slab: 16 MFMAs, the two chains interleaved
-  auto scores = [&](const char* pair, f32x16& s, f32x16& dp) {
+  // S^T and dP^T of one slab: 16 MFMAs, the two chains interleaved.  `between(ks)` runs behind the matrix instructions
+  // of operand step ks: the place for the global -> LDS copies a step owes, which take a wave tens of cycles each to issue.
+  auto scores = [&](const char* pair, f32x16& s, f32x16& dp, auto between) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) { s[r] = 0.f; dp[r] = 0.f; }
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
       s = mfma32(lds_read_b128(pair, rm.rd[ks]), qreg[ks], s);
       dp = mfma32(lds_read_b128(pair + kSlabBytes, rm.rd[ks]), doreg[ks], dp);
+      between(ks);
     }
   };
 
@@ -141,14 +148,33 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     int e_cmp = 0, rem_cmp = nsub;  // list entry of the slab being computed (tile lists: its predicate bits)
     int bits_cmp = kTiled ? idx[0] & 255 : 255;
 
+    // The copies a step requests (K and V slab t+4 into the buffer of slab t, free behind the step's barrier) are issued
+    // by the following step, with block lists in between its first matrix instructions.  Every step requests them, so
+    // that the counter of copies in flight means the same thing at every wait; past the end of the list they repeat a
+    // listed slab into a buffer that nobody reads any more.
+    uint32_t owed_dst = 0;
+    int64_t owed_off = 0;
+
     // step t (t % 4 == R): S_t, dP_t | dS_t | dQ += K_t^T dS_t
-    auto step = [&](auto ring_c, int t) {
+    auto step = [&](auto ring_c, auto first_c, int t) {
       constexpr int R = decltype(ring_c)::value;
+      constexpr bool kOwed = !decltype(first_c)::value;  // the first step owes nothing
       const bool active = !kTiled || (bits_cmp & group_bit) != 0;
+      if constexpr (kTiled && kOwed) {
+        dma.copy(owed_dst, kp + owed_off);
+        dma.copy(owed_dst + kSlabBytes, vp + owed_off);
+      }
       // a wave whose two 16-row groups are both switched off for this slab has nothing to add (wave-uniform branch)
       if (!kTiled || (bits_cmp & wave_bits) != 0) {
         f32x16 s_cur, dp_cur;
-        scores(smem + R * kPairBytes, s_cur, dp_cur);
+        scores(smem + R * kPairBytes, s_cur, dp_cur, [&](int ks) {
+          if constexpr (!kTiled && kOwed) {
+            if (ks == 0) dma.copy_piece(0, owed_dst, kp + owed_off);
+            if (ks == 1) dma.copy_piece(1, owed_dst, kp + owed_off);
+            if (ks == 2) dma.copy_piece(0, owed_dst + kSlabBytes, vp + owed_off);
+            if (ks == 3) dma.copy_piece(1, owed_dst + kSlabBytes, vp + owed_off);
+          }
+        });
         bf16x8 dsk[2];
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
@@ -177,18 +203,22 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
           bits_cmp = e_cmp < cnt ? idx[e_cmp] & 255 : 0;
         }
       }
-      // slab t+2 must have landed (first read in step t+1); the four copies of slab t+3 may still fly
-      if (t + 3 < nsteps) wait_vmem<4>(); else wait_vmem<0>();
+      // slab t+2 must have landed; the four copies of slab t+3 may still fly
+      wait_vmem<4>();
       __syncthreads();
-      if (t + 4 < nsteps) copy_next(R);
+      owed_dst = ring_dst + R * kPairBytes;
+      owed_off = next_off();
     };
-    for (int t = 0; t < nsteps; t += 4) {  // nsteps is even
-      step(IC<0>{}, t);
-      step(IC<1>{}, t + 1);
+    step(IC<0>{}, std::true_type{}, 0);
+    step(IC<1>{}, std::false_type{}, 1);
+    for (int t = 2; t < nsteps; t += 4) {  // nsteps is even
+      step(IC<2>{}, std::false_type{}, t);
+      step(IC<3>{}, std::false_type{}, t + 1);
       if (t + 2 >= nsteps) break;
-      step(IC<2>{}, t + 2);
-      step(IC<3>{}, t + 3);
+      step(IC<0>{}, std::false_type{}, t + 2);
+      step(IC<1>{}, std::false_type{}, t + 3);
     }
+    wait_vmem<0>();  // no copy may still be writing LDS when the work-group gives it back
   }
 
   if (parts > 1) {  // part of a split item: unscaled fp32 partial sums go to the workspace

@@ -202,6 +202,10 @@ struct SlabDma {
     dma16(slab_lds + wave_dst, src, off[0]);
     dma16(slab_lds + wave_dst + 4 * kRowBytes, src, off[1]);
   }
+  // the two halves of copy(), for callers that spread them out
+  FBA_DEVICE void copy_piece(int i, uint32_t slab_lds, const char* src) const {
+    dma16(slab_lds + wave_dst + i * 4 * kRowBytes, src, off[i]);
+  }
 };
 
 // The same copy for the two slabs (K, V) a step of a query-major kernel brings in, by the kWaves waves of its work-group.
