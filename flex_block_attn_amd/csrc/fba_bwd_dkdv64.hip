@@ -170,7 +170,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     const int64_t pair_bytes = (int64_t)p.q_block * p.k_block * 2;
     const int nsub_k = p.k_block / kSlab;
     const int t_key = 4 * ((kt * TK - kblk * p.k_block) / TK) + 2 * kg;  // this wave's first 32-key slab inside the key block
-    const int ho_off0 = ds_unit_store_off(0, lane), ho_off1 = ds_unit_store_off(1, lane);
+    const uint32_t ho_off0 = (uint32_t)ds_unit_store_off(0, lane), ho_off1 = (uint32_t)ds_unit_store_off(1, lane);
     // The common step (the next pair lies in the same query block) is a handful of scalar additions; what the step adds is
     // kept in variables that turn to zero once every listed pair has been requested, so that the cursor then stays on the
     // last pair without a test of its own.
@@ -369,7 +369,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
           s[0][4 * j + e] = pv;
         }
         if constexpr (kHandOver && kExtras) {  // scores() runs only while the wave has a further slab, so ds_unit is set
-          __builtin_nontemporal_store(dsk[j >> 1][j & 1], reinterpret_cast<bf16x8*>(ds_unit + (j >> 1) * 4 * kDsUnitBytes + ((j & 1) ? ho_off1 : ho_off0)));
+          store16_stream(ds_unit + (j >> 1) * 4 * kDsUnitBytes, (j & 1) ? ho_off1 : ho_off0, dsk[j >> 1][j & 1]);
         }
         __builtin_amdgcn_sched_barrier(0);
         da = da_n; db = db_n; va0 = va0_n; va1 = va1_n; vb0 = vb0_n; vb1 = vb1_n; l4 = l4_n;
@@ -479,8 +479,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
       char* ds_unit = reinterpret_cast<char*>(p.ds_ws) + unit_cur;
 #pragma unroll
       for (int grp = 0; grp < 2; ++grp) {
-        __builtin_nontemporal_store(dsk[grp][0], reinterpret_cast<bf16x8*>(ds_unit + grp * 4 * kDsUnitBytes + ho_off0));
-        __builtin_nontemporal_store(dsk[grp][1], reinterpret_cast<bf16x8*>(ds_unit + grp * 4 * kDsUnitBytes + ho_off1));
+        store16_stream(ds_unit + grp * 4 * kDsUnitBytes, ho_off0, dsk[grp][0]);
+        store16_stream(ds_unit + grp * 4 * kDsUnitBytes, ho_off1, dsk[grp][1]);
       }
     }
     // ... and its share of dV, dK (the arithmetic of this call runs on stale registers and is dropped)

@@ -171,6 +171,15 @@ FBA_DEVICE void dma16_stream(uint32_t lds_base, const char* gbase, uint32_t lane
                : "m0");
 }
 
+// Streaming 16-byte store per lane to gbase + lane_off with the base in scalar registers: the compiler forms 64-bit
+// addresses per lane for such a store (a vector add and twice the address traffic per store), which a wave alone on its
+// SIMD pays for.  gbase must be wave-uniform.  Like the copies above the store is tracked by the vector-memory counter
+// only; the compiler does not know of it, so the caller orders it against whatever reads the data (nothing inside the
+// kernels that use it).
+FBA_DEVICE void store16_stream(char* gbase, uint32_t lane_off, bf16x8 value) {
+  asm volatile("global_store_dwordx4 %0, %1, %2 nt" : : "v"(lane_off), "v"(value), "s"(gbase));
+}
+
 // Same for 4 bytes per lane (lane l's dword lands at lds_base + 4 l).
 FBA_DEVICE void dma4(uint32_t lds_base, const char* gbase, uint32_t lane_off) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
