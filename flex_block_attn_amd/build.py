@@ -58,10 +58,68 @@ def _compile_one(src, verbose):
     return obj, log
 
 
+# Sources whose accumulating matrix instructions are inline asm (accumulation-register form).  The compiler gives a
+# matrix instruction of its own the wait states it needs behind a vector instruction that writes one of its operands;
+# an inline-asm one gets none and then reads what the register held before.  The sources keep such writes away from
+# those instructions (opaque pins); this check reads the compiler's assembly of our own kernels and fails the build if a
+# schedule ever brings one within `ASM_HAZARD_WINDOW` instructions again.
+ASM_MFMA_SOURCES = ["fba_bwd_dkdv64.hip"]
+ASM_HAZARD_WINDOW = 4
+
+
+def find_asm_mfma_hazards(asm_text, window=ASM_HAZARD_WINDOW):
+    """[(writer, matrix instruction, distance)] for every vector instruction that writes a register which an
+    accumulation-register matrix instruction at most `window` instructions later reads as operand A or B."""
+    import re
+
+    def regs(tok):
+        m = re.match(r"v\[(\d+):(\d+)\]$", tok)
+        if m:
+            return set(range(int(m.group(1)), int(m.group(2)) + 1))
+        m = re.match(r"v(\d+)$", tok)
+        return {int(m.group(1))} if m else set()
+
+    ins = []
+    for line in asm_text.split("\n"):
+        t = line.strip()
+        if not t or t.startswith(";") or t.startswith("."):
+            continue  # comments, directives and labels (a block may be fallen into, so labels do not end the search)
+        ins.append(t)
+    found = []
+    for i, t in enumerate(ins):
+        if not (t.startswith("v_mfma") and " a[" in t):
+            continue
+        ops = [o.strip() for o in t.split(None, 1)[1].split(",")]
+        src = regs(ops[1]) | regs(ops[2])
+        for back in range(1, window + 1):
+            if i - back < 0:
+                break
+            w = ins[i - back]
+            if w.startswith("v_") and not w.startswith("v_mfma") and not w.startswith("v_accvgpr_read") and " " in w:
+                if regs(w.split(None, 1)[1].split(",")[0].strip()) & src:
+                    found.append((w, t, back))
+    return found
+
+
+def check_asm_mfma_hazards():
+    """Compiles the sources with inline-asm matrix instructions to assembly and raises if a hazard is found."""
+    for src in ASM_MFMA_SOURCES:
+        cmd = [_hipcc(), *HIPCC_FLAGS, *EXTRA_FLAGS.get(src, []), "-S", "--cuda-device-only", os.path.join(CSRC, src), "-o", "-"]
+        r = subprocess.run(cmd, capture_output=True, text=True)
+        if r.returncode != 0:
+            raise RuntimeError(f"hipcc -S failed for {src}:\n{r.stderr[-2000:]}")
+        found = find_asm_mfma_hazards(r.stdout)
+        if found:
+            lines = "\n".join(f"  {w}   ->   {m} (distance {d})" for w, m, d in found)
+            raise RuntimeError(f"{src}: a vector instruction writes an operand of an inline-asm matrix instruction right in front of it:\n{lines}")
+
+
 def build_library(verbose=False):
     """Compile every HIP source and link libfba_gfx950.so. Returns the library path."""
     with concurrent.futures.ThreadPoolExecutor(max_workers=4) as ex:
+        check = ex.submit(check_asm_mfma_hazards)
         results = list(ex.map(lambda s: _compile_one(s, verbose), SOURCES))
+        check.result()
     if verbose:
         for _, log in results:
             if log:

@@ -283,7 +283,9 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     // so the interleaving is written out: one accumulating matrix instruction, then the arithmetic of one accumulator
     // element of both products, each anchored in place.
     f32x16 s[2], dp[2];
-    bf16x8 pk[2][2], dsk[2][2];  // P and dS of the previous slab, packed as B operands
+    // P and dS of a slab, packed as B operands.  Two sets: the slab that is accumulated reads one while the arithmetic of
+    // the next slab fills the other, so that no value has to be moved when a slab is done (the loop below is unrolled by two).
+    bf16x8 pk[2][2][2], dsk[2][2][2];  // [set][key group][16-query step]
 
     // S, dP of the slab in the buffer at byte offset `so` against this wave's 64 keys: every Q / dO operand feeds both key
     // groups.  S comes first, so that while the matrix pipe works on dP the vector unit can already turn S of the first key
@@ -292,8 +294,9 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     // Matrix instructions go in fours, two operand steps each; the operands of the next four are requested before a four
     // is issued, and the scheduling fences keep the compiler from moving the requests back next to their use, where the
     // wave would wait for every fetch.
-    auto scores = [&](auto extras_c, int so, uint32_t req_dst, int64_t req_row, char* ds_unit) {
-      constexpr bool kExtras = decltype(extras_c)::value;  // false for the wave's first slab: nothing to copy or store yet
+    auto scores = [&](auto extras_c, auto set_c, int so, uint32_t req_dst, int64_t req_row, char* ds_unit) {
+      constexpr bool kExtras = decltype(extras_c)::value;
+      constexpr int kSet = decltype(set_c)::value;  // the set that holds dS of the slab to store  // false for the wave's first slab: nothing to copy or store yet
       // accumulator element 4g + e of half-wave h is query row 8g + 4h + e of the slab; dP starts from -delta of its row
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -369,7 +372,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
           s[0][4 * j + e] = pv;
         }
         if constexpr (kHandOver && kExtras) {  // scores() runs only while the wave has a further slab, so ds_unit is set
-          store16_stream(ds_unit + (j >> 1) * 4 * kDsUnitBytes, (j & 1) ? ho_off1 : ho_off0, dsk[j >> 1][j & 1]);
+          store16_stream(ds_unit + (j >> 1) * 4 * kDsUnitBytes, (j & 1) ? ho_off1 : ho_off0, dsk[kSet][j >> 1][j & 1]);
         }
         __builtin_amdgcn_sched_barrier(0);
         da = da_n; db = db_n; va0 = va0_n; va1 = va1_n; vb0 = vb0_n; vb1 = vb1_n; l4 = l4_n;
@@ -380,7 +383,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     // slab (buffer at `po`, operands pk / dsk).  Eight groups of four
     // matrix instructions (one transposed dO operand and one transposed Q operand, each against both key groups) and four
     // accumulator elements of arithmetic; the operands and statistics of group n+1 are requested before group n starts.
-    auto softmax_and_accumulate = [&](int so, int po) {
+    auto softmax_and_accumulate = [&](auto in_c, int so, int po) {
+      constexpr int kIn = decltype(in_c)::value;  // set of the slab that is accumulated; the new P, dS go to the other
       bf16x2 pw[2][8], dw[2][8];  // new P and dS, packed: [key group][register pair]
       LdsPtr ts = t_base + po;
       asm volatile("" : "+v"(ts));
@@ -408,10 +412,10 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
         float pv[4], dsv[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          if (e == 0) mfma32_acc(acc_v[0][mb], adv, pk[0][j]);
-          if (e == 1) mfma32_acc(acc_v[1][mb], adv, pk[1][j]);
-          if (e == 2) mfma32_acc(acc_k[0][mb], adk, dsk[0][j]);
-          if (e == 3) mfma32_acc(acc_k[1][mb], adk, dsk[1][j]);
+          if (e == 0) mfma32_acc(acc_v[0][mb], adv, pk[kIn][0][j]);
+          if (e == 1) mfma32_acc(acc_v[1][mb], adv, pk[kIn][1][j]);
+          if (e == 2) mfma32_acc(acc_k[0][mb], adk, dsk[kIn][0][j]);
+          if (e == 3) mfma32_acc(acc_k[1][mb], adk, dsk[kIn][1][j]);
           pv[e] = grp == 0 ? s[0][4 * g + e] : fast_exp2(__builtin_fmaf(s[1][4 * g + e], c, -l4[e]));
           dsv[e] = pv[e] * dp[grp][4 * g + e];
           if (e & 1) {
@@ -431,9 +435,9 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
       for (int grp = 0; grp < 2; ++grp)
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
-          pk[grp][j] = cat(__builtin_shufflevector(pw[grp][4 * j + 0], pw[grp][4 * j + 1], 0, 1, 2, 3),
+          pk[1 - kIn][grp][j] = cat(__builtin_shufflevector(pw[grp][4 * j + 0], pw[grp][4 * j + 1], 0, 1, 2, 3),
                            __builtin_shufflevector(pw[grp][4 * j + 2], pw[grp][4 * j + 3], 0, 1, 2, 3));
-          dsk[grp][j] = cat(__builtin_shufflevector(dw[grp][4 * j + 0], dw[grp][4 * j + 1], 0, 1, 2, 3),
+          dsk[1 - kIn][grp][j] = cat(__builtin_shufflevector(dw[grp][4 * j + 0], dw[grp][4 * j + 1], 0, 1, 2, 3),
                             __builtin_shufflevector(dw[grp][4 * j + 2], dw[grp][4 * j + 3], 0, 1, 2, 3));
         }
     };
@@ -444,14 +448,23 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 #pragma unroll
       for (int j = 0; j < 2; ++j)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) { pk[grp][j][e] = (__bf16)0.f; dsk[grp][j][e] = (__bf16)0.f; }
-    scores(std::false_type{}, 0, 0, 0, nullptr);
-    // Iteration t: slab t lives in buffer t % 3, slab t-1 in (t+2) % 3, slab t+1 in (t+1) % 3.  The first iteration adds
-    // nothing (P = dS = 0 against the finite rows of slab 0).  The loop body has no branch but the cursor's change of block;
-    // the wave's last slab is handled behind the loop.
+        for (int e = 0; e < 8; ++e) { pk[0][grp][j][e] = (__bf16)0.f; dsk[0][grp][j][e] = (__bf16)0.f; }
+    // The zeros are written here and now (an opaque pin: the compiler cannot put them off or form them again later).
+    // Left to itself it writes them right in front of the first accumulating matrix instruction, which, being inline asm,
+    // gets none of the wait states the compiler gives a matrix instruction that reads a register the vector unit has
+    // just written, and then multiplies by whatever the registers held before.
+#pragma unroll
+    for (int grp = 0; grp < 2; ++grp)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) asm volatile("" : "+v"(pk[0][grp][j]), "+v"(dsk[0][grp][j]));
+    scores(std::false_type{}, IC<0>{}, 0, 0, 0, nullptr);
+    // Iteration t: slab t lives in buffer t % 3, slab t-1 in (t+2) % 3, slab t+1 in (t+1) % 3; P, dS of slab t-1 in set
+    // t % 2.  The first iteration adds nothing (P = dS = 0 against the finite rows of slab 0).  An iteration has no branch
+    // but the cursor's change of block; the wave's last slab is handled behind the loop.
     int cur = 0, prev = 0, nxt = kStageBytes;
-    for (int t = 0; t + 1 < nlocal; ++t) {
-      softmax_and_accumulate(cur, prev);
+    auto iteration = [&](auto in_c) {
+      constexpr int kIn = decltype(in_c)::value;
+      softmax_and_accumulate(in_c, cur, prev);
       char* ds_unit = nullptr;  // where dS_t goes
       if constexpr (kHandOver) ds_unit = reinterpret_cast<char*>(p.ds_ws) + unit_cur;
       // slab t+2 will replace slab t-1 (past the end of the lists: a repeat of the last slab that nobody reads); its copies
@@ -468,23 +481,39 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
       __syncthreads();  // everybody is done with slab t-1 and everybody's copies of slab t+1 have landed
       const int freed = nxt + kStageBytes == 3 * kStageBytes ? 0 : nxt + kStageBytes;  // buffer of slab t-1 = buffer of slab t+2
       const uint32_t req_dst = ring_dst + 3 * par * kStageBytes + freed;
-      scores(std::true_type{}, nxt, req_dst, req_row, ds_unit);
+      scores(std::true_type{}, IC<1 - kIn>{}, nxt, req_dst, req_row, ds_unit);
       prev = cur;
       cur = nxt;
       nxt = freed;
+    };
+    // The compiler zeroes the accumulation registers where it likes, possibly right in front of the first matrix
+    // instruction that adds to them, and does not know that those instructions (inline asm) read them: every accumulator
+    // is pinned here, written, and a few wait states separate the writes from the first read.
+#pragma unroll
+    for (int grp = 0; grp < 2; ++grp)
+#pragma unroll
+      for (int mb = 0; mb < 4; ++mb) {
+        asm volatile("" : "+a"(acc_v[grp][mb]));
+        asm volatile("" : "+a"(acc_k[grp][mb]));
+      }
+    asm volatile("s_nop 7");
+    iteration(IC<0>{});  // nlocal is even and at least 2: iterations 0 .. nlocal-2, an odd number of them
+    for (int t = 1; t + 1 < nlocal; t += 2) {
+      iteration(IC<1>{});
+      iteration(IC<0>{});
     }
-    // the wave's last slab: no scores() follows that could carry its dS stores
-    softmax_and_accumulate(cur, prev);
+    // the wave's last slab (an odd one): no scores() follows that could carry its dS stores
+    softmax_and_accumulate(IC<1>{}, cur, prev);
     if constexpr (kHandOver) {
       char* ds_unit = reinterpret_cast<char*>(p.ds_ws) + unit_cur;
 #pragma unroll
       for (int grp = 0; grp < 2; ++grp) {
-        store16_stream(ds_unit + grp * 4 * kDsUnitBytes, ho_off0, dsk[grp][0]);
-        store16_stream(ds_unit + grp * 4 * kDsUnitBytes, ho_off1, dsk[grp][1]);
+        store16_stream(ds_unit + grp * 4 * kDsUnitBytes, ho_off0, dsk[0][grp][0]);
+        store16_stream(ds_unit + grp * 4 * kDsUnitBytes, ho_off1, dsk[0][grp][1]);
       }
     }
     // ... and its share of dV, dK (the arithmetic of this call runs on stale registers and is dropped)
-    softmax_and_accumulate(nxt, cur);
+    softmax_and_accumulate(IC<0>{}, nxt, cur);
     wait_vmem<0>();
     __syncthreads();  // no copy is writing LDS any more; V and the ring are free
 

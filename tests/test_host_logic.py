@@ -327,3 +327,20 @@ def test_no_alloc_backward_rejects_oversized_problems(lib):
     f = _fake()
     rc = h.fba_bwd_noalloc(*([f] * 13), 1, 1, 64, 64, 128 * 1024, 128 * 1024, 128, 128, 128, _null())
     assert rc == lib.FBA_ERR_UNSUPPORTED and b"exceed the built-in workspace" in h.fba_last_error()
+
+
+def test_build_check_finds_a_write_in_front_of_an_asm_matrix_instruction():
+    """build.find_asm_mfma_hazards: a vector instruction that writes an A / B operand of an accumulation-register matrix
+    instruction at most a few instructions earlier is reported, also across a label (the block may be fallen into);
+    writes of other registers, writes further away and the compiler's own (vector-register) matrix instructions are not."""
+    from flex_block_attn_amd.build import find_asm_mfma_hazards
+
+    mfma = "v_mfma_f32_32x32x16_bf16 a[224:239], v[54:57], v[50:53], a[224:239]"
+    bad = "\n".join(["v_mov_b64_e32 v[50:51], s[40:41]", "s_waitcnt lgkmcnt(6)", mfma])
+    assert [(w.split()[0], d) for w, _m, d in find_asm_mfma_hazards(bad)] == [("v_mov_b64_e32", 2)]
+    assert find_asm_mfma_hazards("\n".join(["v_cvt_pk_bf16_f32 v57, v1, v2", mfma]))[0][2] == 1
+    assert find_asm_mfma_hazards("\n".join(["v_mov_b32_e32 v58, 0", "ds_read_b64_tr_b16 v[54:55], v9", mfma])) == []
+    far = "\n".join(["v_mov_b32_e32 v50, 0"] + ["s_nop 0"] * 4 + [mfma])
+    assert find_asm_mfma_hazards(far) == []
+    assert len(find_asm_mfma_hazards("\n".join(["v_mov_b32_e32 v50, 0", ".LBB0_7:", mfma]))) == 1
+    assert find_asm_mfma_hazards("\n".join(["v_mov_b32_e32 v50, 0", "v_mfma_f32_32x32x16_bf16 v[0:15], v[54:57], v[50:53], v[0:15]"])) == []
