@@ -328,22 +328,16 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
           l4 = lds_read_f32x4(st_ptr + so);
         }
         __builtin_amdgcn_sched_barrier(0);
-        // the copies of the slab after next are issued one at a time between the matrix instructions (copies first, the dS
-        // stores of the slab before last: the wait before the next barrier then lets the four youngest operations, the
-        // stores, stay in flight)
+        // the copies of the slab after next are issued one at a time behind every second matrix instruction (vector-memory
+        // instructions that follow each other closely cost the wave more), the last one in the dP part ahead of the first
+        // dS store: copies first, stores last, so that the wait before the next barrier lets the four youngest
+        // operations, the stores, stay in flight
         s[0] = mfma32(qa, kreg[0][2 * j], s[0]);
-        if constexpr (kExtras) {
-          if (j < 3) issue_copy_part(3 * j, req_dst, req_row);
-        }
         s[1] = mfma32(qa, kreg[1][2 * j], s[1]);
-        if constexpr (kExtras) {
-          if (j < 3) issue_copy_part(3 * j + 1, req_dst, req_row);
-        }
+        if constexpr (kExtras) issue_copy_part(2 * j, req_dst, req_row);
         s[0] = mfma32(qb, kreg[0][2 * j + 1], s[0]);
-        if constexpr (kExtras) {
-          if (j < 3) issue_copy_part(3 * j + 2, req_dst, req_row);
-        }
         s[1] = mfma32(qb, kreg[1][2 * j + 1], s[1]);
+        if constexpr (kExtras) issue_copy_part(2 * j + 1, req_dst, req_row);
         __builtin_amdgcn_sched_barrier(0);
         qa = qa_n; qb = qb_n;
       }
@@ -364,6 +358,9 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           if (e == 0) dp[0] = mfma32(da, va0, dp[0]);
+          if constexpr (kExtras) {
+            if (e == 1 && j == 0) issue_copy_part(8, req_dst, req_row);
+          }
           if (e == 1) dp[1] = mfma32(da, va1, dp[1]);
           if (e == 2) dp[0] = mfma32(db, vb0, dp[0]);
           if (e == 3) dp[1] = mfma32(db, vb1, dp[1]);
