@@ -219,7 +219,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     const int64_t pair_bytes = (int64_t)p.q_block * p.k_block * 2;
     const int nsub_k = p.k_block / kSlab;
     const int t_key = 4 * ((kt * TK - kblk * p.k_block) / TK) + kg;  // this wave's 32-key slab inside the key block
-    const int ho_off0 = ds_unit_store_off(0, lane), ho_off1 = ds_unit_store_off(1, lane);
+    const uint32_t ho_off0 = (uint32_t)ds_unit_store_off(0, lane), ho_off1 = (uint32_t)ds_unit_store_off(1, lane);
     auto ho_next_entry = [&]() {
       ++h_e;
       while (h_e >= h_cnt) {
@@ -318,8 +318,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
           unit += (h_slot0 + h_e) * pair_bytes + ((int64_t)((h_s >> 2) * nsub_k + t_key) * 4 + (h_s & 3)) * kDsUnitBytes;
         // written once, read once by another kernel much later: streaming stores, so that they do not push the Q / dO
         // slabs that other work-groups are about to fetch out of L2
-        __builtin_nontemporal_store(dsk[0], reinterpret_cast<bf16x8*>(unit + ho_off0));
-        __builtin_nontemporal_store(dsk[1], reinterpret_cast<bf16x8*>(unit + ho_off1));
+        store16_stream(unit, ho_off0, dsk[0]);
+        store16_stream(unit, ho_off1, dsk[1]);
       }
 #pragma unroll
       for (int j = 0; j < 2; ++j)
