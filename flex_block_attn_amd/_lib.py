@@ -39,7 +39,7 @@ SIGNATURES = {
     "fba_block_mean": (_c_i32, [_c_ptr, _c_ptr, _c_i64, _c_i32, _c_i32, _c_i32, _c_ptr]),
     "fba_ssta_mask": (_c_i32, [_c_ptr, _c_ptr, _c_ptr, _c_ptr] + [_c_i32] * 10 + [_c_ptr]),
     "fba_tile_permute": (_c_i32, [_c_ptr, _c_ptr, _c_i64] + [_c_i32] * 8 + [_c_ptr]),
-    "fba_fwd_tiled": (_c_i32, [_c_ptr] * 7 + [_c_i64] + [_c_i32] * 8 + [_c_ptr]),
+    "fba_fwd_tiled": (_c_i32, [_c_ptr] * 7 + [_c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
     "fba_bwd_tiled": (_c_i32, [_c_ptr] * 14 + [_c_i64] + [_c_i32] * 8 + [_c_ptr]),
     "fba_bwd_stats": (_c_i32, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i32, _c_ptr]),
     "fba_bwd_dq": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),

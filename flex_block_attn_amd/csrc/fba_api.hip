@@ -79,7 +79,7 @@ int check_split_ws(const void* ws, int64_t bytes) {
 
 extern "C" {
 
-int32_t fba_version(void) { return 2001; }
+int32_t fba_version(void) { return 2002; }
 
 const char* fba_last_error(void) { return g_err; }
 
@@ -148,8 +148,9 @@ int32_t fba_fwd(const void* q, const void* k, const void* v, void* o, float* lse
 
 int32_t fba_fwd_tiled(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* qt_cnt,
                       const int32_t* qt_ent, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
-                      int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
-  return fwd_impl(q, k, v, o, lse, qt_cnt, qt_ent, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, nullptr, 0, hip_stream, true);
+                      int32_t head_dim, int32_t q_block, int32_t k_block, void* split_ws, int64_t split_ws_bytes,
+                      void* hip_stream) {
+  return fwd_impl(q, k, v, o, lse, qt_cnt, qt_ent, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block, split_ws, split_ws_bytes, hip_stream, true);
 }
 
 int32_t fba_block_mean(const void* x, float* out, int64_t n_seq, int32_t S, int32_t block, int32_t head_dim, void* hip_stream) {

@@ -238,9 +238,9 @@ __global__ __attribute__((amdgpu_flat_work_group_size(64 * kWaves, 64 * kWaves),
 
     bf16x8 p_prev[2];
     // predicate of the slab whose softmax is next (tile lists): all 16-row groups share the entry, each lane tests its bit
-    int e_cmp = 0, rem_cmp = nsub;
-    int bits_cmp = kTiled ? idx[0] & 255 : 255;
-    int bits_ahead = kTiled && cnt > 1 ? idx[1] & 255 : 0;  // predicate bits of the following list entry
+    int e_cmp = e_begin, rem_cmp = nsub - sub_begin;
+    int bits_cmp = kTiled ? idx[e_begin] & 255 : 255;
+    int bits_ahead = kTiled && e_begin + 1 < cnt ? idx[e_begin + 1] & 255 : 0;  // predicate bits of the following list entry
     // A wave whose two 16-row groups are both switched off for a slab leaves that slab's matrix work out altogether
     // (wave-uniform branches); rows switched off inside an active wave are dealt with by selects.
     const int wave_bits = 3 << (2 * wave);
@@ -388,8 +388,8 @@ hipError_t launch_fwd(FwdParams p, hipStream_t stream) {
   void (*fn)(const FwdParams) = p.tiled ? &fwd_kernel<true, 4> : wide ? &fwd_kernel<false, 12> : &fwd_kernel<false, 4>;
   const int rows = wide ? 384 : 128;
   p.num_items = p.B * p.Hq * (p.Sq / rows);
-  // tail splitting for the 128-row kernel on block lists (two work-groups per compute unit)
-  p.split = plan_split(p.num_items, 2, kFwdSlotBytes, (p.tiled || wide) ? nullptr : p.split.ws, p.split_ws_bytes);
+  // tail splitting for the 128-row kernels (two work-groups per compute unit)
+  p.split = plan_split(p.num_items, 2, kFwdSlotBytes, wide ? nullptr : p.split.ws, p.split_ws_bytes);
   plan_xcd_mapping(p.B * p.Hq, p.split.first, p.items_per_xcd, p.split.main_wgs);
   const int split_wgs = (p.num_items - p.split.first) * p.split.parts;
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);

@@ -243,11 +243,8 @@ def forward_with_lists(q, k, v, q_block_size, kv_block_size, lists):
     args = (_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(lse), _ptr(lists.q_cnt), _ptr(lists.q_idx), lists.mask_bh,
             B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size)
     with torch.cuda.device(q.device):
-        if lists.tiled:
-            _lib.call("fba_fwd_tiled", *args, _stream())
-        else:
-            _ws, ws_ptr, ws_bytes = _split_workspace(q.device)
-            _lib.call("fba_fwd", *args, ws_ptr, ws_bytes, _stream())
+        _ws, ws_ptr, ws_bytes = _split_workspace(q.device)
+        _lib.call("fba_fwd_tiled" if lists.tiled else "fba_fwd", *args, ws_ptr, ws_bytes, _stream())
     return o, lse
 
 

@@ -63,7 +63,7 @@ int32_t fba_mask_compact(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32
  *                   the call's work on the stream; its contents before and after are meaningless
  *   split_ws_bytes  its size; fba_split_workspace_bytes() is what the planner can use at most (a smaller buffer limits
  *                   the number of ranges, never correctness)
- * Block lists only: the _tiled entry points do not split.
+ * Block lists, and forward on tile lists: the other _tiled entry points do not split.
  */
 int64_t fba_split_workspace_bytes(void);
 
@@ -173,7 +173,8 @@ int32_t fba_tile_lists(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32_t
                        int32_t* qt_cnt, int32_t* qt_ent, int32_t* kt_cnt, int32_t* kt_ent, void* hip_stream);
 int32_t fba_fwd_tiled(const void* q, const void* k, const void* v, void* o, float* lse, const int32_t* qt_cnt,
                       const int32_t* qt_ent, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv,
-                      int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+                      int32_t head_dim, int32_t q_block, int32_t k_block,
+                      void* split_ws, int64_t split_ws_bytes, void* hip_stream);
 int32_t fba_bwd_tiled(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                       float* stats, void* dq, void* dk, void* dv, const int32_t* qt_cnt, const int32_t* qt_ent,
                       const int32_t* kt_cnt, const int32_t* kt_ent, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,

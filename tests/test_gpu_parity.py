@@ -832,6 +832,38 @@ def test_measurement_variants_give_the_same_bits(gpu, cfg, monkeypatch):
                 assert torch.equal(a, b)
 
 
+def test_tile_list_forward_splits_its_tail(oracle, gpu, monkeypatch):
+    """Forward on tile lists with and without the splitting workspace: a launch smaller than the GPU (every tile cut into
+    parts) against the oracle, and a launch of 2.25 rounds (the last quarter round cut into parts) against itself without
+    splitting; entries switched off for some 16-row groups, an empty query block and a range that starts inside an entry's
+    second slab are all in there."""
+    import flex_block_attn_amd as fba
+    from flex_block_attn_amd import interface
+
+    g = torch.Generator(device="cpu").manual_seed(31)
+    m = torch.rand((1, 2, 12, 6), generator=g) < 0.5
+    m[..., 3, :] = False
+    for split in (None, "0"):
+        monkeypatch.setattr(interface, "SPLIT_WORKSPACE_MIB", split)
+        _run_case(oracle, gpu, 1, 2, 2, 768, 384, 64, 64, m, seed=32)
+    B, H, S, bs = 1, 9, 16384, 64  # 1152 tiles of 128 rows on 512 slots
+    nb = S // bs
+    q, k, v = (torch.randn((B, H, S, 128), generator=g).to(torch.bfloat16).to(gpu) for _ in range(3))
+    mask = (torch.rand((B, H, nb, nb), generator=g) < 0.15).to(gpu)
+    lists = fba.lists_for(mask, bs, bs)
+    assert lists.tiled
+    outs = []
+    for split in (None, "0"):
+        monkeypatch.setattr(interface, "SPLIT_WORKSPACE_MIB", split)
+        outs.append(fba.forward_with_lists(q, k, v, bs, bs, lists))
+    (o_a, lse_a), (o_b, lse_b) = outs
+    assert not torch.equal(o_a[:, -1], o_b[:, -1])  # the last tiles did sum in another order
+    assert torch.equal(o_a[:, 0], o_b[:, 0]) and torch.equal(lse_a[:, 0], lse_b[:, 0])
+    assert (o_a.float() - o_b.float()).abs().max().item() <= 2e-2
+    both = torch.isfinite(lse_a) & torch.isfinite(lse_b)
+    assert torch.equal(torch.isfinite(lse_a), torch.isfinite(lse_b)) and (lse_a[both] - lse_b[both]).abs().max().item() <= 1e-3
+
+
 def test_backward_memory_follows_the_sequence_length(gpu):
     """One head, S=30720, all 80 x 80 blocks of 384: the dS of that head (1.9 GB) is more than the default backward may
     allocate (six times the call's own tensors), so it recomputes instead and its peak allocation stays within twice the

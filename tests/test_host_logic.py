@@ -68,9 +68,9 @@ def test_c_abi_argument_validation(lib):
     assert fwd(1, 1, 2, 2, 256, 256, 128, 64, 128) == lib.FBA_ERR_UNSUPPORTED
     assert b"q_block" in h.fba_last_error()
     # ... and the tile-list entry points take it, as long as the sequence lengths are multiples of 128
-    assert h.fba_fwd_tiled(f, f, f, f, f, f, f, 1, 1, 2, 2, 192, 192, 128, 64, 64, _null()) == lib.FBA_ERR_UNSUPPORTED
+    assert h.fba_fwd_tiled(f, f, f, f, f, f, f, 1, 1, 2, 2, 192, 192, 128, 64, 64, _null(), 0, _null()) == lib.FBA_ERR_UNSUPPORTED
     assert b"multiples of 128" in h.fba_last_error()
-    assert h.fba_fwd_tiled(_null(), f, f, f, f, f, f, 1, 1, 2, 2, 256, 256, 128, 64, 64, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_fwd_tiled(_null(), f, f, f, f, f, f, 1, 1, 2, 2, 256, 256, 128, 64, 64, _null(), 0, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_tile_lists(f, 1, 3, 3, 64, 64, f, f, f, f, _null()) == lib.FBA_ERR_UNSUPPORTED
     assert h.fba_tile_lists(f, 1, 4, 4, 24, 64, f, f, f, f, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_tile_lists(f, 1, 4, 4, 64, 64, f, _null(), f, f, _null()) == lib.FBA_ERR_INVALID
