@@ -372,6 +372,7 @@ int32_t fba_bwd_dkdv_handover(const void* q, const void* k, const void* v, const
   p.q = (const __bf16*)q; p.k = (const __bf16*)k; p.v = (const __bf16*)v; p.d_o = (const __bf16*)d_o;
   p.stats = stats; p.dk = (__bf16*)dk; p.dv = (__bf16*)dv; p.k_cnt = k_cnt; p.k_idx = k_idx;
   p.ds_ws = (__bf16*)ds_ws; p.pair_base = pair_base;
+  p.ws_pairs = ds_ws_bytes / ((int64_t)q_block * k_block * 2);
   p.split.ws = (float*)split_ws; p.split_ws_bytes = split_ws_bytes;
   hipError_t e = launch_dkdv_variant(p, (hipStream_t)hip_stream);
   return e == hipSuccess ? FBA_OK : hip_fail(e, "dkdv (hand-over) launch");
@@ -391,6 +392,7 @@ int32_t fba_bwd_dq_from_ds(const void* k, const void* ds_ws, int64_t ds_ws_bytes
   fill_bwd(p, s);
   p.k = (const __bf16*)k; p.dq = (__bf16*)dq; p.q_cnt = q_cnt; p.q_idx = q_idx;
   p.ds_ws = (__bf16*)const_cast<void*>(ds_ws); p.pair_base = pair_base; p.q_slot = q_slot;
+  p.ws_pairs = ds_ws_bytes / ((int64_t)q_block * k_block * 2);
   p.split.ws = (float*)split_ws; p.split_ws_bytes = split_ws_bytes;
   hipError_t e = fba::launch_bwd_dq_from_ds(p, (hipStream_t)hip_stream);
   return e == hipSuccess ? FBA_OK : hip_fail(e, "dq (from dS) launch");
@@ -454,6 +456,7 @@ int32_t fba_bwd_tiled_handover(const void* q, const void* k, const void* v, cons
   p.stats = stats; p.dq = (__bf16*)dq; p.dk = (__bf16*)dk; p.dv = (__bf16*)dv;
   p.q_cnt = qt_cnt; p.q_idx = qt_ent; p.k_cnt = kt_cnt; p.k_idx = kt_ent;
   p.ds_ws = (__bf16*)ds_ws; p.pair_base = pair_base; p.k_slot = kt_slot; p.q_slot = slot_table;
+  p.ws_pairs = ds_ws_bytes / (128 * 128 * 2);
   hipError_t e = fba::launch_bwd_dkdv(p, (hipStream_t)hip_stream);
   if (e != hipSuccess) return hip_fail(e, "dkdv (tile lists, hand-over) launch");
   e = fba::launch_bwd_dq_from_ds(p, (hipStream_t)hip_stream);

@@ -50,6 +50,9 @@ template <bool kTiled, bool kHandOver>
 __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_per_eu(2, 2))) void dkdv_kernel(const BwdParams p) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int TK = 128;
+  if constexpr (kHandOver) {
+    if (!workspace_holds_lists(p)) return;  // the launcher's last launch reports it
+  }
 
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -419,7 +422,11 @@ hipError_t launch_bwd_dkdv(BwdParams p, hipStream_t stream) {
     const int64_t row0 = (int64_t)p.split.first * 128;
     e = launch_partial_sum(p.split.ws, p.split.parts, 2 * 128 * kHeadDim, p.dv, row0, split_items, 1.f, stream);
     if (e != hipSuccess) return e;
-    return launch_partial_sum(p.split.ws + 128 * kHeadDim, p.split.parts, 2 * 128 * kHeadDim, p.dk, row0, split_items, p.scale, stream);
+    e = launch_partial_sum(p.split.ws + 128 * kHeadDim, p.split.parts, 2 * 128 * kHeadDim, p.dk, row0, split_items, p.scale, stream);
+    if (e != hipSuccess) return e;
+  }
+  if (hand_over) {
+    return launch_poison_unless_fit(p, p.dk, p.dv, (int64_t)p.B * p.Hkv * p.Skv * kHeadDim, stream);
   }
   return hipGetLastError();
 }

@@ -53,7 +53,6 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   constexpr bool kTiled = false;
   extern __shared__ __attribute__((aligned(16))) char smem[];
   constexpr int TK = 128;
-
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kg = wave & 1, par = wave >> 1;  // 64-key group, slab parity
@@ -86,6 +85,11 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   int slabs_all = 0;
   for (int g = 0; g < group; ++g) slabs_all += k_cnt[list_row(g)];
   slabs_all *= nsub;
+  if constexpr (kHandOver) {
+    // lists that number more pairs than the workspace holds: no slab is touched, nothing is stored into the workspace
+    // (the launcher's last launch then reports it)
+    if (!workspace_holds_lists(p)) slabs_all = 0;
+  }
   // this work-group's range of listed slabs: all of them, or part `part` of `parts` (boundaries on multiples of four slabs;
   // block lists only)
   const int s_begin = parts == 1 ? 0 : 4 * (int)(((int64_t)(slabs_all / 4) * part) / parts);
@@ -170,7 +174,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     const int64_t pair_bytes = (int64_t)p.q_block * p.k_block * 2;
     const int nsub_k = p.k_block / kSlab;
     const int t_key = 4 * ((kt * TK - kblk * p.k_block) / TK) + 2 * kg;  // this wave's first 32-key slab inside the key block
-    const uint32_t ho_off0 = (uint32_t)ds_unit_store_off(0, lane), ho_off1 = (uint32_t)ds_unit_store_off(1, lane);
+    const uint32_t ho_off0 = (uint32_t)ds_unit_store_off(0, lane);  // the second chunk's offset is formed from it at the store
     // The common step (the next pair lies in the same query block) is a handful of scalar additions; what the step adds is
     // kept in variables that turn to zero once every listed pair has been requested, so that the cursor then stays on the
     // last pair without a test of its own.
@@ -234,10 +238,11 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
       dma4(dst + 2 * kSlabBytes, stbase + row * 4, stat_off);  // both waves copy the same 256 bytes
     };
     // the same request one copy at a time (i = 0..8), for spreading over a phase of matrix instructions
+    uint32_t stat_off_loop = stat_off;
     auto issue_copy_part = [&](int i, uint32_t dst, int64_t row) {
       if (i < 4) dma16(dst + dma_dst + i * 4 * kRowBytes, qbase + row * kRowBytes, dma_off[i]);
       else if (i < 8) dma16(dst + kSlabBytes + dma_dst + (i - 4) * 4 * kRowBytes, dobase + row * kRowBytes, dma_off[i - 4]);
-      else dma4(dst + 2 * kSlabBytes, stbase + row * 4, stat_off);
+      else dma4(dst + 2 * kSlabBytes, stbase + row * 4, stat_off_loop);
     };
     // A parity keeps three buffers: ring buffer 3 * par + (i % 3) holds its slab of pair i.
     if (parts == 1) {
@@ -257,6 +262,9 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
     advance();
     wait_vmem<0>();
     __syncthreads();
+    // a value of its own from here on: held in one register through the loop instead of being fetched back from the
+    // spill area wherever the compiler had cut the kernel-long live range
+    asm volatile("" : "+v"(stat_off_loop));
 
     // Per-lane fetch addresses with the wave's share folded in: slab addresses carry the parity's three buffers, V
     // addresses the wave's 64 keys.  One register each: the operand step (row-major fetches) and the column block and row
@@ -369,7 +377,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
           s[0][4 * j + e] = pv;
         }
         if constexpr (kHandOver && kExtras) {  // scores() runs only while the wave has a further slab, so ds_unit is set
-          store16_stream(ds_unit + (j >> 1) * 4 * kDsUnitBytes, (j & 1) ? ho_off1 : ho_off0, dsk[kSet][j >> 1][j & 1]);
+          if (j & 1) store16_stream_second(ds_unit + (j >> 1) * 4 * kDsUnitBytes, ho_off0, dsk[kSet][j >> 1][1]);
+          else store16_stream(ds_unit + (j >> 1) * 4 * kDsUnitBytes, ho_off0, dsk[kSet][j >> 1][0]);
         }
         __builtin_amdgcn_sched_barrier(0);
         da = da_n; db = db_n; va0 = va0_n; va1 = va1_n; vb0 = vb0_n; vb1 = vb1_n; l4 = l4_n;
@@ -506,7 +515,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 #pragma unroll
       for (int grp = 0; grp < 2; ++grp) {
         store16_stream(ds_unit + grp * 4 * kDsUnitBytes, ho_off0, dsk[0][grp][0]);
-        store16_stream(ds_unit + grp * 4 * kDsUnitBytes, ho_off1, dsk[0][grp][1]);
+        store16_stream_second(ds_unit + grp * 4 * kDsUnitBytes, ho_off0, dsk[0][grp][1]);
       }
     }
     // ... and its share of dV, dK (the arithmetic of this call runs on stale registers and is dropped)
@@ -586,7 +595,11 @@ hipError_t launch_bwd_dkdv64(BwdParams p, hipStream_t stream) {
     const int64_t row0 = (int64_t)p.split.first * 128;
     e = launch_partial_sum(p.split.ws, p.split.parts, 2 * 128 * kHeadDim, p.dv, row0, split_items, 1.f, stream);
     if (e != hipSuccess) return e;
-    return launch_partial_sum(p.split.ws + 128 * kHeadDim, p.split.parts, 2 * 128 * kHeadDim, p.dk, row0, split_items, p.scale, stream);
+    e = launch_partial_sum(p.split.ws + 128 * kHeadDim, p.split.parts, 2 * 128 * kHeadDim, p.dk, row0, split_items, p.scale, stream);
+    if (e != hipSuccess) return e;
+  }
+  if (p.ds_ws != nullptr) {
+    return launch_poison_unless_fit(p, p.dk, p.dv, (int64_t)p.B * p.Hkv * p.Skv * kHeadDim, stream);
   }
   return hipGetLastError();
 }

@@ -42,6 +42,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   extern __shared__ __attribute__((aligned(16))) char smem[];  // ring [4] of (K slab | dS units)
   constexpr int TQ = 128;
 
+  if (!workspace_holds_lists(p)) return;  // the launcher's last launch reports it
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // whole items first (dealt to the XCDs in contiguous spans), then the parts of the split items
@@ -266,6 +267,22 @@ hipError_t launch_partial_sum(const float* ws, int parts, int64_t slot_floats, _
   return hipGetLastError();
 }
 
+__global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void poison_unless_fit_kernel(const BwdParams p, __bf16* __restrict__ out_a, __bf16* __restrict__ out_b, int64_t n) {
+  if (workspace_holds_lists(p)) return;
+  const __bf16 nan = (__bf16)__builtin_nanf("");
+  for (int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x; t < n; t += (int64_t)gridDim.x * 256) {
+    out_a[t] = nan;
+    if (out_b) out_b[t] = nan;
+  }
+}
+
+hipError_t launch_poison_unless_fit(const BwdParams& p, __bf16* out_a, __bf16* out_b, int64_t n, hipStream_t stream) {
+  if (n <= 0) return hipSuccess;
+  const int64_t blocks = (n + 255) / 256;
+  hipLaunchKernelGGL(poison_unless_fit_kernel, dim3((unsigned)(blocks < 2048 ? blocks : 2048)), dim3(256), 0, stream, p, out_a, out_b, n);
+  return hipGetLastError();
+}
+
 hipError_t launch_bwd_dq_from_ds(BwdParams p, hipStream_t stream) {
   constexpr int kSmem = kRing * kStageBytes;
   if (p.ds_ws == nullptr) return hipErrorInvalidValue;
@@ -280,9 +297,11 @@ hipError_t launch_bwd_dq_from_ds(BwdParams p, hipStream_t stream) {
   e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmem);
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(fn, dim3(p.split.main_wgs + split_items * p.split.parts), dim3(256), kSmem, stream, p);
-  if (split_items > 0)
-    return launch_partial_sum(p.split.ws, p.split.parts, 128 * kHeadDim, p.dq, (int64_t)p.split.first * 128, split_items, p.scale, stream);
-  return hipGetLastError();
+  if (split_items > 0) {
+    e = launch_partial_sum(p.split.ws, p.split.parts, 128 * kHeadDim, p.dq, (int64_t)p.split.first * 128, split_items, p.scale, stream);
+    if (e != hipSuccess) return e;
+  }
+  return launch_poison_unless_fit(p, p.dq, nullptr, (int64_t)p.B * p.Hq * p.Sq * kHeadDim, stream);
 }
 
 }  // namespace fba

@@ -180,6 +180,16 @@ FBA_DEVICE void store16_stream(char* gbase, uint32_t lane_off, bf16x8 value) {
   asm volatile("global_store_dwordx4 %0, %1, %2 nt" : : "v"(lane_off), "v"(value), "s"(gbase));
 }
 
+// The same store to gbase + (lane_off ^ 128) + 1024: where a lane's second offset differs from its first in bit 7 and by
+// 1024 (ds_unit_store_off(1, lane) against ds_unit_store_off(0, lane)), it is formed here from the first instead of being
+// held in a register of its own for the whole kernel.
+FBA_DEVICE void store16_stream_second(char* gbase, uint32_t lane_off, bf16x8 value) {
+  uint32_t second;
+  asm volatile("v_xor_b32 %0, 128, %1\n\tglobal_store_dwordx4 %0, %2, %3 offset:1024 nt"
+               : "=&v"(second)
+               : "v"(lane_off), "v"(value), "s"(gbase));
+}
+
 // Same for 4 bytes per lane (lane l's dword lands at lds_base + 4 l).
 FBA_DEVICE void dma4(uint32_t lds_base, const char* gbase, uint32_t lane_off) {
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
@@ -330,5 +340,16 @@ FBA_DEVICE int ds_unit_slot_off(int key, int u) {
 // 32-query slab 4 tq + w of the query block against 32-key slab t of the key block, so a 128-row query tile tq reads its
 // whole share of the pair as one ascending stream, 8 KiB (four units, one per wave) per 32-key step.
 constexpr int kDsUnitBytes = 2048;
+
+// Do the pairs that the lists of a hand-over call number fit the workspace?  P is BwdParams: pair_base holds the exclusive
+// prefix sums of the rows this call covers (rows + 1 entries); the workspace pointer is where pair 0 would live, the call
+// touches the pairs from pair_base[0] up to pair_base[rows], once per (batch, head) when all share one mask.
+template <typename P>
+FBA_DEVICE bool workspace_holds_lists(const P& p) {
+  const ConstIdx pb = const_idx(p.pair_base);
+  const int64_t rows = p.mask_bh * (p.tiled ? p.Skv / 128 : p.nK);
+  const int64_t listed = (int64_t)(pb[rows] - pb[0]) * (p.mask_bh == 1 ? (int64_t)p.B * p.Hq : 1);
+  return listed <= p.ws_pairs;
+}
 
 }  // namespace fba

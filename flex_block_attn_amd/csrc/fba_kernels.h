@@ -97,6 +97,7 @@ struct BwdParams {
   //   q_slot    [mask_bh, Sq/128, Skv/128]:     pair number of (query tile, key tile), -1 where nothing is listed
   //   zero_unit: 2 KiB of zeros in device memory, read in place of a dS unit that no wave stored
   __bf16* ds_ws;
+  int64_t ws_pairs;  // pairs ds_ws has room for
   const int32_t* pair_base;
   const int32_t* q_slot;
   const int32_t* k_slot;
@@ -121,6 +122,11 @@ hipError_t launch_bwd_dq(BwdParams p, hipStream_t stream);
 hipError_t launch_bwd_dkdv(BwdParams p, hipStream_t stream);
 hipError_t launch_bwd_dkdv64(BwdParams p, hipStream_t stream);  // block lists only: 64 keys per wave, one wave per SIMD
 hipError_t launch_bwd_dq_from_ds(BwdParams p, hipStream_t stream);
+// The lists of a hand-over call live in device memory, so only kernels can tell whether the pairs they number fit the
+// workspace.  Every kernel that stores or fetches dS tests it first (workspace_holds_lists, fba_common.h) and returns at
+// once when they do not; this launch then fills `n` bf16 values at `out_a` (and at `out_b` unless null) with NaN, so that
+// the call fails loudly instead of writing out of bounds.
+hipError_t launch_poison_unless_fit(const BwdParams& p, __bf16* out_a, __bf16* out_b, int64_t n, hipStream_t stream);
 hipError_t launch_partial_sum(const float* ws, int parts, int64_t slot_floats, __bf16* out, int64_t out_row0, int n_items, float scale,
                               hipStream_t stream);
 hipError_t launch_probe_mfma(const float* src, float* sink, int work_groups, int iters, hipStream_t stream);

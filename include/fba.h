@@ -115,10 +115,12 @@ int32_t fba_bwd_dkdv(const void* q, const void* k, const void* v, const void* d_
  *                    number of pairs in the lists), q_slot [mask_bh, nQ, nK] = the pair number of every q_idx entry
  *                    (-1 beyond q_cnt).
  *   ds_ws            n_pairs * q_block * k_block bf16, 16-byte aligned; n_pairs = selected pairs over all (batch,
- *                    head): the sum of k_cnt, times B * Hq when mask_bh == 1.  ds_ws_bytes is its size; the caller
- *                    vouches that n_pairs matches the lists (they live in device memory and are not read back): the
- *                    kernels address ds_ws by the pair numbers in pair_base / q_slot, so lists that do not belong to
- *                    this n_pairs and workspace make them write out of bounds.
+ *                    head): the sum of k_cnt, times B * Hq when mask_bh == 1.  ds_ws_bytes is its size.  The lists live
+ *                    in device memory and are not read back, so the host cannot tell whether they belong to this
+ *                    n_pairs; the kernels can: the call touches the pairs from pair_base[0] up to the last entry of
+ *                    pair_base (times B * Hq when mask_bh == 1), and if ds_ws_bytes does not hold that many, no kernel
+ *                    stores or fetches any dS and dq, dk, dv come back filled with NaN (the return code stays FBA_OK).
+ *                    q_slot must come from the same fba_pair_slots call as pair_base.
  * Every head's dS is independent: a caller short of memory may run these entry points once per group of kv heads through
  * one smaller workspace, with all pointers moved to the group's first head (B = 1) and ds_ws moved back by the pairs in
  * front of the group when the mask is per head (the pair numbers in the lists are absolute).
@@ -191,7 +193,8 @@ int32_t fba_bwd_tiled(const void* q, const void* k, const void* v, const void* o
  *                   [mask_bh, Sq/128, Skv/128] = pair number of (query tile, key tile), -1 where nothing is listed.
  *                   n_qt = Sq/128, n_kt = Skv/128.
  *   ds_ws           n_pairs * 32 KiB, 16-byte aligned; n_pairs = listed tile pairs over all (batch, head): the last
- *                   entry of pair_base, times B * Hq when mask_bh == 1.  The caller vouches that n_pairs matches the lists.
+ *                   entry of pair_base, times B * Hq when mask_bh == 1.  As for fba_bwd_handover, lists that number more
+ *                   pairs than ds_ws_bytes holds leave the workspace untouched and dq, dk, dv filled with NaN.
  * Other arguments as fba_bwd_tiled; dk, dv agree with fba_bwd_tiled's bit for bit, dq to within bf16 rounding of dS.
  */
 int32_t fba_tile_slots(const int32_t* kt_cnt, const int32_t* kt_ent, int64_t mask_bh, int32_t n_qt, int32_t n_kt, int32_t* pair_base,

@@ -864,6 +864,52 @@ def test_tile_list_forward_splits_its_tail(oracle, gpu, monkeypatch):
     assert torch.equal(torch.isfinite(lse_a), torch.isfinite(lse_b)) and (lse_a[both] - lse_b[both]).abs().max().item() <= 1e-3
 
 
+@pytest.mark.parametrize("bs", [128, 64])
+def test_handover_with_a_workspace_too_small_for_the_lists_fails_loudly(gpu, bs):
+    """A hand-over call whose lists number more pairs than the workspace is said to hold (lists rebuilt, a stale pair
+    count): the host cannot see it, the kernels can.  Nothing is stored into the workspace and dQ, dK, dV come back as
+    NaN; the same call with the true size gives what backward_with_lists gives.  Block lists and tile lists."""
+    import ctypes
+
+    import flex_block_attn_amd as fba
+    from flex_block_attn_amd import _lib, interface
+    from flex_block_attn_amd.interface import _ptr, _stream
+
+    B, H, S = 1, 3, 1024
+    g = torch.Generator(device="cpu").manual_seed(41 + bs)
+    q, k, v, do = (torch.randn((B, H, S, 128), generator=g).to(torch.bfloat16).to(gpu) for _ in range(4))
+    mask = (torch.rand((B, H, S // bs, S // bs), generator=g) < 0.5).to(gpu)
+    lists = fba.lists_for(mask, bs, bs)
+    assert lists.tiled == (bs == 64)
+    o, lse = fba.forward_with_lists(q, k, v, bs, bs, lists)
+    want = fba.backward_with_lists(q, k, v, o, lse, do, bs, bs, lists, hand_over=True)
+    pairs, ws_bytes = interface.ds_workspace_bytes(lists, B, H, bs, bs)
+    pair_bytes = ws_bytes // pairs
+    ws = torch.full((ws_bytes,), 0x5A, dtype=torch.uint8, device=gpu)  # full size, so that nothing could leave the allocation
+    stats = torch.empty((2, B, H, S), dtype=torch.float32, device=gpu)
+    _split, sp_ptr, sp_bytes = interface._split_workspace(q.device)  # as backward_with_lists: same tiles split, same sums
+
+    def call(n_pairs):
+        dq, dk, dv = (torch.zeros_like(t) for t in (q, k, v))
+        head = (_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), _ptr(ws), n_pairs * pair_bytes,
+                _ptr(dq), _ptr(dk), _ptr(dv), _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx))
+        shape = (n_pairs, lists.mask_bh, B, H, H, S, S, 128, bs, bs)
+        if lists.tiled:
+            _lib.call("fba_bwd_tiled_handover", *head, _ptr(lists.pair_base), _ptr(lists.k_slot), _ptr(lists.q_slot), *shape, _stream())
+        else:
+            _lib.call("fba_bwd_handover", *head, _ptr(lists.pair_base), _ptr(lists.q_slot), *shape, sp_ptr, sp_bytes, _stream())
+        torch.cuda.synchronize()
+        return dq, dk, dv
+
+    for short in (pairs - 1, pairs // 2):
+        got = call(short)
+        for t in got:
+            assert torch.isnan(t).all()
+        assert (ws == 0x5A).all()
+    for a, b in zip(call(pairs), want):
+        assert torch.equal(a, b)
+
+
 def test_backward_memory_follows_the_sequence_length(gpu):
     """One head, S=30720, all 80 x 80 blocks of 384: the dS of that head (1.9 GB) is more than the default backward may
     allocate (six times the call's own tensors), so it recomputes instead and its peak allocation stays within twice the
