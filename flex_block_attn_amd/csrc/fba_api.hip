@@ -173,7 +173,7 @@ int32_t fba_ssta_mask(const float* q_mean, const float* k_mean, const uint8_t* b
   if (q_block <= 0 || k_block <= 0) return fail(FBA_ERR_INVALID, "q_block and k_block must be positive");
   if (topk < 0 || band < -1 || sink < 0) return fail(FBA_ERR_INVALID, "topk, sink must be >= 0 and band >= -1 (got %d %d %d)", topk, sink, band);
   if (!q_mean || !k_mean || !mask) return fail(FBA_ERR_INVALID, "null pointer argument");
-  if (nK > 1024) return fail(FBA_ERR_UNSUPPORTED, "at most 1024 key blocks are ranked per query block (got %d)", nK);
+  if (nK > 4096) return fail(FBA_ERR_UNSUPPORTED, "at most 4096 key blocks are ranked per query block (got %d)", nK);
   if ((int64_t)B * Hq > 65535) return fail(FBA_ERR_UNSUPPORTED, "B*Hq (%lld) must be at most 65535", (long long)B * Hq);
   hipError_t e = fba::launch_ssta_mask(q_mean, k_mean, base, mask, (int64_t)B * Hq, Hq, Hkv, nQ, nK, q_block, k_block, topk, band,
                                        sink, (hipStream_t)hip_stream);

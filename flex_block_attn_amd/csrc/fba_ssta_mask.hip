@@ -53,11 +53,13 @@ constexpr int kQPerWave = 2;
 constexpr int kQPerGroup = 8;      // query blocks per work-group (4 waves x 2)
 constexpr int kChunk = 64;         // key blocks per LDS chunk: one per lane
 constexpr int kRowStride = kD + 1; // floats; lane-per-row reads hit 64 different banks
-constexpr int kMaxChunks = 16;     // nK <= 1024
+constexpr int kChunksSmall = 16;   // nK <= 1024: 32 score registers per lane
+constexpr int kChunksLarge = 64;   // nK <= 4096: 128 score registers per lane
 
 // mask[bh, i, j] = (j among the topk largest <q_mean[bh,i], k_mean[kv(bh),j]>, ties to the lower j)
 //                  || |j - (i*q_block)/k_block| <= band || j < sink || base[i, j]   (base: optional [nQ, nK] mask).
-// A wave ranks two query blocks; lane l holds the scores of key blocks l, l+64, ... in registers.
+// A wave ranks two query blocks; lane l holds the scores of key blocks l, l+64, ... (kMaxChunks of them) in registers.
+template <int kMaxChunks>
 __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void ssta_mask_kernel(
     const float* __restrict__ q_mean, const float* __restrict__ k_mean, const uint8_t* __restrict__ base,
     uint8_t* __restrict__ mask, int Hq, int Hkv, int nQ, int nK, int q_block, int k_block, int topk, int band, int sink) {
@@ -104,7 +106,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void ssta_mask
   for (int qq = 0; qq < kQPerWave; ++qq) {
     const int i = i0 + wave * kQPerWave + qq;
     if (i >= nQ) break;  // uniform over the wave
-    uint32_t sel = 0;
+    uint64_t sel = 0;
     for (int round = 0; round < topk; ++round) {
       float best = ninf;
       int bt = -1;
@@ -125,7 +127,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void ssta_mask
         }
       }
       if (j == 0x7fffffff) break;  // nothing left to pick: every lane sees the same j
-      if ((j & 63) == lane) sel |= 1u << (j >> 6);
+      if ((j & 63) == lane) sel |= 1ull << (j >> 6);
     }
     const int diag = (int)(((int64_t)i * q_block) / k_block);
     uint8_t* row = mask + (size_t)(bh * nQ + i) * nK;
@@ -135,7 +137,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void ssta_mask
       if (j < nK) {
         const int dist = j > diag ? j - diag : diag - j;
         const uint32_t keep = base ? (base[(size_t)i * nK + j] != 0) : 0u;
-        row[j] = (uint8_t)(((sel >> t) & 1u) | (dist <= band) | (j < sink) | keep);
+        row[j] = (uint8_t)((uint32_t)((sel >> t) & 1u) | (dist <= band) | (j < sink) | keep);
       }
     }
   }
@@ -174,8 +176,10 @@ hipError_t launch_block_mean(const __bf16* x, float* out, int64_t n_blocks, int 
 
 hipError_t launch_ssta_mask(const float* q_mean, const float* k_mean, const uint8_t* base, uint8_t* mask, int64_t BH, int Hq, int Hkv, int nQ,
                             int nK, int q_block, int k_block, int topk, int band, int sink, hipStream_t stream) {
-  if (BH <= 0 || BH > 65535 || nK > kChunk * kMaxChunks) return hipErrorInvalidValue;
-  hipLaunchKernelGGL(ssta_mask_kernel, dim3((unsigned)((nQ + kQPerGroup - 1) / kQPerGroup), (unsigned)BH), dim3(256), 0,
+  if (BH <= 0 || BH > 65535 || nK > kChunk * kChunksLarge) return hipErrorInvalidValue;
+  void (*fn)(const float*, const float*, const uint8_t*, uint8_t*, int, int, int, int, int, int, int, int, int) =
+      nK <= kChunk * kChunksSmall ? &ssta_mask_kernel<kChunksSmall> : &ssta_mask_kernel<kChunksLarge>;
+  hipLaunchKernelGGL(fn, dim3((unsigned)((nQ + kQPerGroup - 1) / kQPerGroup), (unsigned)BH), dim3(256), 0,
                      stream, q_mean, k_mean, base, mask, Hq, Hkv, nQ, nK, q_block, k_block, topk, band, sink);
   return hipGetLastError();
 }

@@ -216,7 +216,7 @@ int32_t fba_bwd_tiled_handover(const void* q, const void* k, const void* v, cons
  * fba_ssta_mask: mask[b, h, i, j] (bool bytes, [B, Hq, nQ, nK]) = j is one of the `topk` key blocks with the largest
  *   <q_mean[b,h,i], k_mean[b, h / (Hq/Hkv), j]> (equal scores: lower j first), or |j - (i*q_block)/k_block| <= band, or
  *   j < sink, or base[i, j] (base: bool bytes [nQ, nK] shared by every (b, h), e.g. a sliding-tile mask; may be null).
- *   band = -1 switches the band off.  nK <= 1024.
+ *   band = -1 switches the band off.  nK <= 4096 (FBA_ERR_UNSUPPORTED beyond).
  * fba_tile_permute: moves 256-byte token rows of x [n_seq, T*H*W, 128] bf16 between raster order of the (T, H, W) grid
  *   and tile order (tiles of tile_t x tile_h x tile_w tokens, tiles in raster order of the tile grid, tokens in raster
  *   order inside a tile), so that one tile is one contiguous block of the attention; to_tiles = 0 is the inverse.

@@ -50,6 +50,8 @@ def test_block_mean(oracle, gpu, block, S):
     (2, 4, 2, 1024, 1024, 128, 128, 4, 1, 1),      # grouped kv heads
     (1, 1, 1, 384 * 70, 384 * 70, 384, 384, 16, 1, 1),   # more than one 64-block chunk of key blocks
     (1, 2, 1, 256, 64 * 200, 128, 64, 16, 0, 0),   # 200 key blocks, moba style
+    (1, 1, 1, 1152, 64 * 1500, 128, 64, 16, 1, 1), # 1500 key blocks: the kernel that ranks up to 4096
+    (1, 1, 1, 256, 64 * 4096, 128, 64, 7, 0, 1),   # the largest number of key blocks it takes
     (1, 1, 1, 512, 512, 128, 128, 9, -1, 0),       # topk beyond the number of key blocks
     (1, 1, 1, 1152, 384, 128, 384, 0, 1, 2),       # nothing ranked: band and sink only
 ])

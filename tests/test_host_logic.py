@@ -93,7 +93,7 @@ def test_c_abi_argument_validation(lib):
     assert h.fba_block_mean(f, f, 4, 256, 64, 64, _null()) == lib.FBA_ERR_INVALID and b"head_dim" in h.fba_last_error()
     assert h.fba_block_mean(_null(), f, 4, 256, 64, 128, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_ssta_mask(f, f, _null(), f, 1, 3, 2, 4, 4, 128, 128, 2, 1, 1, _null()) == lib.FBA_ERR_INVALID
-    assert h.fba_ssta_mask(f, f, _null(), f, 1, 2, 2, 4, 2000, 128, 128, 2, 1, 1, _null()) == lib.FBA_ERR_UNSUPPORTED
+    assert h.fba_ssta_mask(f, f, _null(), f, 1, 2, 2, 4, 5000, 128, 128, 2, 1, 1, _null()) == lib.FBA_ERR_UNSUPPORTED
     assert h.fba_ssta_mask(f, f, _null(), _null(), 1, 2, 2, 4, 4, 128, 128, 2, 1, 1, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_ssta_mask(f, f, _null(), f, 1, 2, 2, 4, 4, 128, 128, -1, 1, 1, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_tile_permute(f, _fake(0x2000), 1, 6, 8, 9, 6, 8, 8, 128, 1, _null()) == lib.FBA_ERR_INVALID and b"divide" in h.fba_last_error()
