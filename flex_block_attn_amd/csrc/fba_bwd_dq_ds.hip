@@ -279,7 +279,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256))) void poison_un
 hipError_t launch_poison_unless_fit(const BwdParams& p, __bf16* out_a, __bf16* out_b, int64_t n, hipStream_t stream) {
   if (n <= 0) return hipSuccess;
   const int64_t blocks = (n + 255) / 256;
-  hipLaunchKernelGGL(poison_unless_fit_kernel, dim3((unsigned)(blocks < 2048 ? blocks : 2048)), dim3(256), 0, stream, p, out_a, out_b, n);
+  hipLaunchKernelGGL(poison_unless_fit_kernel, dim3((unsigned)(blocks < 64 ? blocks : 64)), dim3(256), 0, stream, p, out_a, out_b, n);
   return hipGetLastError();
 }
 
