@@ -33,14 +33,14 @@ SIGNATURES = {
     "fba_bwd_dkdv_handover": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_ptr] * 3 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
     "fba_bwd_dq_from_ds": (_c_i32, [_c_ptr] * 2 + [_c_i64] + [_c_ptr] * 5 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
     "fba_tile_slots": (_c_i32, [_c_ptr, _c_ptr, _c_i64, _c_i32, _c_i32, _c_ptr, _c_ptr, _c_ptr, _c_ptr]),
-    "fba_bwd_tiled_handover": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_ptr] * 10 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr]),
+    "fba_bwd_tiled_handover": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_ptr] * 10 + [_c_i64, _c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
     "fba_bwd_noalloc": (_c_i32, [_c_ptr] * 13 + [_c_i64] + [_c_i32] * 8 + [_c_ptr]),
     "fba_tile_lists": (_c_i32, [_c_ptr, _c_i64, _c_i32, _c_i32, _c_i32, _c_i32, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_ptr]),
     "fba_block_mean": (_c_i32, [_c_ptr, _c_ptr, _c_i64, _c_i32, _c_i32, _c_i32, _c_ptr]),
     "fba_ssta_mask": (_c_i32, [_c_ptr, _c_ptr, _c_ptr, _c_ptr] + [_c_i32] * 10 + [_c_ptr]),
     "fba_tile_permute": (_c_i32, [_c_ptr, _c_ptr, _c_i64] + [_c_i32] * 8 + [_c_ptr]),
     "fba_fwd_tiled": (_c_i32, [_c_ptr] * 7 + [_c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
-    "fba_bwd_tiled": (_c_i32, [_c_ptr] * 14 + [_c_i64] + [_c_i32] * 8 + [_c_ptr]),
+    "fba_bwd_tiled": (_c_i32, [_c_ptr] * 14 + [_c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
     "fba_bwd_stats": (_c_i32, [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_i64, _c_i32, _c_ptr]),
     "fba_bwd_dq": (_c_i32, [_c_ptr] * 8 + [_c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
     "fba_bwd_dkdv": (_c_i32, [_c_ptr] * 9 + [_c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),

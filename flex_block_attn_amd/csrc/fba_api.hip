@@ -79,7 +79,7 @@ int check_split_ws(const void* ws, int64_t bytes) {
 
 extern "C" {
 
-int32_t fba_version(void) { return 2002; }
+int32_t fba_version(void) { return 2003; }
 
 const char* fba_last_error(void) { return g_err; }
 
@@ -434,10 +434,11 @@ int32_t fba_bwd_tiled_handover(const void* q, const void* k, const void* v, cons
                                const int32_t* qt_ent, const int32_t* kt_cnt, const int32_t* kt_ent, const int32_t* pair_base,
                                const int32_t* kt_slot, const int32_t* slot_table, int64_t n_pairs, int64_t mask_bh, int32_t B,
                                int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,
-                               void* hip_stream) {
+                               void* split_ws, int64_t split_ws_bytes, void* hip_stream) {
   const Shape s{mask_bh, B, Hq, Hkv, Sq, Skv, head_dim, q_block, k_block};
   if (int rc = check_shape(s)) return rc;
   if (int rc = check_lists(s, true, "backward")) return rc;
+  if (int rc = check_split_ws(split_ws, split_ws_bytes)) return rc;
   // everything is validated before the first launch, so that a rejected call leaves nothing on the stream
   if (int rc = check_ptrs({{"q", q}, {"k", k}, {"v", v}, {"o", o}, {"d_o", d_o}, {"dq", dq}, {"dk", dk}, {"dv", dv}, {"ds_ws", ds_ws}})) return rc;
   if (!lse || !stats || !qt_cnt || !qt_ent || !kt_cnt || !kt_ent || !pair_base || !kt_slot || !slot_table)
@@ -457,6 +458,7 @@ int32_t fba_bwd_tiled_handover(const void* q, const void* k, const void* v, cons
   p.q_cnt = qt_cnt; p.q_idx = qt_ent; p.k_cnt = kt_cnt; p.k_idx = kt_ent;
   p.ds_ws = (__bf16*)ds_ws; p.pair_base = pair_base; p.k_slot = kt_slot; p.q_slot = slot_table;
   p.ws_pairs = ds_ws_bytes / (128 * 128 * 2);
+  p.split.ws = (float*)split_ws; p.split_ws_bytes = split_ws_bytes;
   hipError_t e = fba::launch_bwd_dkdv(p, (hipStream_t)hip_stream);
   if (e != hipSuccess) return hip_fail(e, "dkdv (tile lists, hand-over) launch");
   e = fba::launch_bwd_dq_from_ds(p, (hipStream_t)hip_stream);
@@ -516,9 +518,10 @@ int32_t fba_bwd_noalloc(const void* q, const void* k, const void* v, const void*
 int32_t fba_bwd_tiled(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                       float* stats, void* dq, void* dk, void* dv, const int32_t* qt_cnt, const int32_t* qt_ent,
                       const int32_t* kt_cnt, const int32_t* kt_ent, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
-                      int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream) {
+                      int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,
+                      void* split_ws, int64_t split_ws_bytes, void* hip_stream) {
   return bwd_impl(q, k, v, o, d_o, lse, stats, dq, dk, dv, qt_cnt, qt_ent, kt_cnt, kt_ent, mask_bh, B, Hq, Hkv, Sq, Skv, head_dim,
-                  q_block, k_block, nullptr, 0, hip_stream, true);
+                  q_block, k_block, split_ws, split_ws_bytes, hip_stream, true);
 }
 
 }  // extern "C"

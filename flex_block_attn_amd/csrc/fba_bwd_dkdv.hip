@@ -86,10 +86,10 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
   int slabs_all = 0;
   for (int g = 0; g < group; ++g) slabs_all += k_cnt[list_row(g)];
   slabs_all *= nsub;
-  // this work-group's range of listed slabs: all of them, or part `part` of `parts` (boundaries on multiples of four slabs;
-  // block lists only)
+  // this work-group's range of listed slabs: all of them, or part `part` of `parts` (boundaries on multiples of four slabs)
   const int s_begin = parts == 1 ? 0 : 4 * (int)(((int64_t)(slabs_all / 4) * part) / parts);
-  const int nslabs = (parts == 1 ? slabs_all : 4 * (int)(((int64_t)(slabs_all / 4) * (part + 1)) / parts)) - s_begin;
+  // (the last part takes what is left over: with tile lists the number of listed slabs need not be a multiple of four)
+  const int nslabs = (part + 1 == parts ? slabs_all : 4 * (int)(((int64_t)(slabs_all / 4) * (part + 1)) / parts)) - s_begin;
   // (query head of the group, list entry, slab inside the query block) of slab s_begin
   int g_begin = 0, e_begin = 0, sub_begin = 0;
   if (parts > 1) {
@@ -179,7 +179,7 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
       idx_cur = const_idx(p.k_idx + lr * row_len);
       head_row0 = ((int64_t)b * p.Hq + hkv * group + g_cur) * p.Sq;
       e_cur = e_begin;
-      row_next = head_row0 + (int64_t)idx_cur[e_cur] * p.q_block + sub_begin * kSlab;
+      row_next = head_row0 + (kTiled ? (int64_t)(idx_cur[e_cur] >> 8) * kSlab : (int64_t)idx_cur[e_cur] * p.q_block + sub_begin * kSlab);
       rem = nsub - sub_begin;
     }
     request_pair(0);
@@ -190,18 +190,21 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
     int g_cmp = -1, e_cmp = -1, cnt_cmp = 0, bits_cmp = 0, sub_cmp = 0;
     int64_t slot_cmp = 0, head_slot0 = 0;
     ConstIdx idx_cmp = nullptr, slot_idx_cmp = nullptr;
+    auto enter_cmp_head = [&]() {  // list row of query head g_cmp of the group
+      const int64_t lr = list_row(g_cmp);
+      cnt_cmp = k_cnt[lr];
+      idx_cmp = const_idx(p.k_idx + lr * row_len);
+      if constexpr (kHandOver) {
+        slot_idx_cmp = const_idx(p.k_slot + lr * row_len);
+        const int64_t bh = (int64_t)b * p.Hq + hkv * group + g_cmp;
+        head_slot0 = p.mask_bh == 1 ? bh * const_idx(p.pair_base)[tiles_per_head] : 0;
+      }
+    };
     auto next_bits = [&]() {
       ++e_cmp;
       while (e_cmp >= cnt_cmp) {
         if (++g_cmp >= group) { bits_cmp = 0; return; }
-        const int64_t lr = list_row(g_cmp);
-        cnt_cmp = k_cnt[lr];
-        idx_cmp = const_idx(p.k_idx + lr * row_len);
-        if constexpr (kHandOver) {
-          slot_idx_cmp = const_idx(p.k_slot + lr * row_len);
-          const int64_t bh = (int64_t)b * p.Hq + hkv * group + g_cmp;
-          head_slot0 = p.mask_bh == 1 ? bh * const_idx(p.pair_base)[tiles_per_head] : 0;
-        }
+        enter_cmp_head();
         e_cmp = 0;
       }
       const int ent = idx_cmp[e_cmp];
@@ -212,6 +215,11 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
       }
     };
     if constexpr (kTiled) {
+      if (parts > 1) {  // start in the middle of the lists, as the cursor of the copies does
+        g_cmp = g_begin;
+        enter_cmp_head();
+        e_cmp = e_begin - 1;
+      }
       next_bits();
       if (par) next_bits();
     }
@@ -408,8 +416,8 @@ __global__ __attribute__((amdgpu_flat_work_group_size(512, 512), amdgpu_waves_pe
 
 hipError_t launch_bwd_dkdv(BwdParams p, hipStream_t stream) {
   p.num_items = p.B * p.Hkv * (p.Skv / 128);
-  // tail splitting on block lists (one work-group per compute unit); a part stores two 128 x 128 fp32 tiles
-  p.split = plan_split(p.num_items, 1, 2 * 128 * kHeadDim * 4, p.tiled ? nullptr : p.split.ws, p.split_ws_bytes);
+  // tail splitting (one work-group per compute unit); a part stores two 128 x 128 fp32 tiles
+  p.split = plan_split(p.num_items, 1, 2 * 128 * kHeadDim * 4, p.split.ws, p.split_ws_bytes);
   plan_xcd_mapping(p.B * p.Hkv, p.split.first, p.items_per_xcd, p.split.main_wgs);
   const int split_items = p.num_items - p.split.first;
   const bool hand_over = p.ds_ws != nullptr;

@@ -385,14 +385,14 @@ def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists,
     group = Hq // Hkv
     M = lists.mask_bh
     with torch.cuda.device(q.device):
-        _ws, sp_ptr, sp_bytes = (None, None, 0) if lists.tiled else _split_workspace(q.device)
+        _ws, sp_ptr, sp_bytes = _split_workspace(q.device)
         if chunks is None:
             stats = torch.empty((2, B, Hq, Sq), dtype=torch.float32, device=q.device)
             common = (_ptr(q), _ptr(k), _ptr(v), _ptr(o), _ptr(do), _ptr(lse), _ptr(stats), _ptr(dq), _ptr(dk), _ptr(dv),
                       _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx), M,
                       B, Hq, Hkv, Sq, Skv, HEAD_DIM, q_block_size, kv_block_size)
             if lists.tiled:
-                _lib.call("fba_bwd_tiled", *common, _stream())
+                _lib.call("fba_bwd_tiled", *common, sp_ptr, sp_bytes, _stream())
             else:
                 _lib.call("fba_bwd", *common, sp_ptr, sp_bytes, _stream())
             return dq, dk, dv
@@ -413,7 +413,7 @@ def backward_with_lists(q, k, v, o, lse, do, q_block_size, kv_block_size, lists,
                     _ptr(stats), ws_ptr, pairs * pair_bytes, _offset(dq, qo), _offset(dk, ko), _offset(dv, ko),
                     _offset(lists.q_cnt, m0 * n_qt), _offset(lists.q_idx, m0 * n_qt * lists.nK), _offset(lists.k_cnt, m0 * n_kt),
                     _offset(lists.k_idx, m0 * n_kt * 4 * n_qt), _offset(lists.pair_base, m0 * n_kt), _offset(lists.k_slot, m0 * n_kt * 4 * n_qt),
-                    _offset(lists.q_slot, m0 * n_qt * n_kt), pairs, *shape, _stream(),
+                    _offset(lists.q_slot, m0 * n_qt * n_kt), pairs, *shape, sp_ptr, sp_bytes, _stream(),
                 )
             else:
                 nQ, nK = lists.nQ, lists.nK

@@ -63,7 +63,7 @@ int32_t fba_mask_compact(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32
  *                   the call's work on the stream; its contents before and after are meaningless
  *   split_ws_bytes  its size; fba_split_workspace_bytes() is what the planner can use at most (a smaller buffer limits
  *                   the number of ranges, never correctness)
- * Block lists, and forward on tile lists: the other _tiled entry points do not split.
+ * On tile lists forward and the dK/dV kernel split; the dQ kernels do not.
  */
 int64_t fba_split_workspace_bytes(void);
 
@@ -180,7 +180,8 @@ int32_t fba_fwd_tiled(const void* q, const void* k, const void* v, void* o, floa
 int32_t fba_bwd_tiled(const void* q, const void* k, const void* v, const void* o, const void* d_o, const float* lse,
                       float* stats, void* dq, void* dk, void* dv, const int32_t* qt_cnt, const int32_t* qt_ent,
                       const int32_t* kt_cnt, const int32_t* kt_ent, int64_t mask_bh, int32_t B, int32_t Hq, int32_t Hkv,
-                      int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block, void* hip_stream);
+                      int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,
+                      void* split_ws, int64_t split_ws_bytes, void* hip_stream);
 
 /*
  * fba_bwd_tiled with dS handed over in memory, as fba_bwd_handover does for block lists (the reference's counterpart
@@ -204,7 +205,7 @@ int32_t fba_bwd_tiled_handover(const void* q, const void* k, const void* v, cons
                                const int32_t* qt_ent, const int32_t* kt_cnt, const int32_t* kt_ent, const int32_t* pair_base,
                                const int32_t* kt_slot, const int32_t* slot_table, int64_t n_pairs, int64_t mask_bh, int32_t B,
                                int32_t Hq, int32_t Hkv, int32_t Sq, int32_t Skv, int32_t head_dim, int32_t q_block, int32_t k_block,
-                               void* hip_stream);
+                               void* split_ws, int64_t split_ws_bytes, void* hip_stream);
 
 /*
  * Callers' side of the operator for video models.  The reference names these steps but never released them

@@ -895,7 +895,7 @@ def test_handover_with_a_workspace_too_small_for_the_lists_fails_loudly(gpu, bs)
                 _ptr(dq), _ptr(dk), _ptr(dv), _ptr(lists.q_cnt), _ptr(lists.q_idx), _ptr(lists.k_cnt), _ptr(lists.k_idx))
         shape = (n_pairs, lists.mask_bh, B, H, H, S, S, 128, bs, bs)
         if lists.tiled:
-            _lib.call("fba_bwd_tiled_handover", *head, _ptr(lists.pair_base), _ptr(lists.k_slot), _ptr(lists.q_slot), *shape, _stream())
+            _lib.call("fba_bwd_tiled_handover", *head, _ptr(lists.pair_base), _ptr(lists.k_slot), _ptr(lists.q_slot), *shape, sp_ptr, sp_bytes, _stream())
         else:
             _lib.call("fba_bwd_handover", *head, _ptr(lists.pair_base), _ptr(lists.q_slot), *shape, sp_ptr, sp_bytes, _stream())
         torch.cuda.synchronize()

@@ -74,16 +74,16 @@ def test_c_abi_argument_validation(lib):
     assert h.fba_tile_lists(f, 1, 3, 3, 64, 64, f, f, f, f, _null()) == lib.FBA_ERR_UNSUPPORTED
     assert h.fba_tile_lists(f, 1, 4, 4, 24, 64, f, f, f, f, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_tile_lists(f, 1, 4, 4, 64, 64, f, _null(), f, f, _null()) == lib.FBA_ERR_INVALID
-    assert h.fba_bwd_tiled(*([f] * 14), 1, 1, 2, 2, 256, 256, 128, 64, 96, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_bwd_tiled(*([f] * 14), 1, 1, 2, 2, 256, 256, 128, 64, 96, _null(), 0, _null()) == lib.FBA_ERR_INVALID
     # tile-pair numbering and the tile-list backward that hands dS over
     assert h.fba_tile_slots(f, f, 0, 2, 2, f, f, f, _null()) == lib.FBA_ERR_INVALID and b"positive" in h.fba_last_error()
     assert h.fba_tile_slots(f, f, 1, 2, 2, f, _null(), f, _null()) == lib.FBA_ERR_INVALID
     tho = [f] * 8 + [2 * 32768] + [f] * 10
-    assert h.fba_bwd_tiled_handover(*tho, 3, 1, 1, 2, 2, 256, 256, 128, 64, 64, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_bwd_tiled_handover(*tho, 3, 1, 1, 2, 2, 256, 256, 128, 64, 64, _null(), 0, _null()) == lib.FBA_ERR_INVALID
     assert b"3 tile pairs" in h.fba_last_error()
-    assert h.fba_bwd_tiled_handover(*tho, 2, 1, 1, 2, 2, 192, 192, 128, 64, 64, _null()) == lib.FBA_ERR_UNSUPPORTED
+    assert h.fba_bwd_tiled_handover(*tho, 2, 1, 1, 2, 2, 192, 192, 128, 64, 64, _null(), 0, _null()) == lib.FBA_ERR_UNSUPPORTED
     tho[18] = _null()  # slot_table
-    assert h.fba_bwd_tiled_handover(*tho, 2, 1, 1, 2, 2, 256, 256, 128, 64, 64, _null()) == lib.FBA_ERR_INVALID
+    assert h.fba_bwd_tiled_handover(*tho, 2, 1, 1, 2, 2, 256, 256, 128, 64, 64, _null(), 0, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_mask_compact(f, 0, 4, 4, f, f, f, f, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_mask_compact(_null(), 1, 4, 4, f, f, f, f, _null()) == lib.FBA_ERR_INVALID
     assert h.fba_bwd_stats(f, f, f, f, 16, 64, _null()) == lib.FBA_ERR_INVALID
