@@ -46,6 +46,9 @@ SIGNATURES = {
     "fba_bwd_dkdv": (_c_i32, [_c_ptr] * 9 + [_c_i64] + [_c_i32] * 8 + [_c_ptr, _c_i64, _c_ptr]),
 }
 
+# fba_version() of the library these signatures describe (include/fba.h; bumped whenever an argument list changes)
+ABI_VERSION = 2003
+
 _lib = None
 
 
@@ -69,6 +72,13 @@ def load():
             "(hipcc, --offload-arch=gfx950). There is no fallback path."
         )
     lib = ctypes.CDLL(LIB_PATH)
+    lib.fba_version.restype = _c_i32
+    lib.fba_version.argtypes = []
+    if lib.fba_version() != ABI_VERSION:  # argument lists below belong to exactly this version
+        raise ImportError(
+            f"{LIB_PATH} reports version {lib.fba_version()}, this package binds version {ABI_VERSION}: "
+            "rebuild it with `python -m flex_block_attn_amd.build`."
+        )
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)
         fn.restype = res

@@ -79,7 +79,7 @@ int check_split_ws(const void* ws, int64_t bytes) {
 
 extern "C" {
 
-int32_t fba_version(void) { return 2003; }
+int32_t fba_version(void) { return FBA_VERSION; }
 
 const char* fba_last_error(void) { return g_err; }
 

@@ -34,7 +34,9 @@ extern "C" {
 #define FBA_ERR_UNSUPPORTED 2 /* valid for the operator, but no kernel variant covers it yet */
 #define FBA_ERR_HIP 3         /* a HIP runtime call failed */
 
-/* Library version: major * 1000 + minor. */
+/* Library version: major * 1000 + minor; the minor number goes up whenever an argument list in this header changes, so a
+ * binding can refuse a library built from another header (flex_block_attn_amd/_lib.py does). */
+#define FBA_VERSION 2003
 int32_t fba_version(void);
 
 /* Message for the last non-OK return on the calling thread ("" if none). The pointer stays valid until the next

@@ -28,7 +28,7 @@ def test_every_declared_symbol_is_exported(lib):
     handle = lib.load()
     for name in declared:
         assert getattr(handle, name) is not None
-    assert handle.fba_version() >= 1000
+    assert handle.fba_version() == lib.ABI_VERSION
 
 
 def _null():
