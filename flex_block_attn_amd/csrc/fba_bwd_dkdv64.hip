@@ -56,13 +56,22 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
   const int tid = threadIdx.x, lane = tid & 63, l32 = lane & 31, h = lane >> 5;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int kg = wave & 1, par = wave >> 1;  // 64-key group, slab parity
+  // the grid index this work-group works on: its own, or one it claims (a launch with claim counters)
+  int grid_index = (int)blockIdx.x;
+  if (p.queue != nullptr) {
+    volatile int* claimed = reinterpret_cast<volatile int*>(smem + kSmemBytes);  // behind everything the kernel uses
+    if (tid == 0) *claimed = claim_work(p.queue, xcd_id(), p.total_work);
+    __syncthreads();
+    grid_index = __builtin_amdgcn_readfirstlane(*claimed);
+    if (grid_index < 0) return;
+  }
   // whole items first (dealt to the XCDs in contiguous spans), then the parts of the split items
   int item, part = 0, parts = 1;
-  if ((int)blockIdx.x < p.split.main_wgs) {
-    item = xcd_remap(blockIdx.x, p.items_per_xcd);
+  if (grid_index < p.split.main_wgs) {
+    item = xcd_remap(grid_index, p.items_per_xcd);
     if (item >= p.split.first) return;
   } else {
-    const int s = blockIdx.x - p.split.main_wgs;
+    const int s = grid_index - p.split.main_wgs;
     item = p.split.first + s / p.split.parts;
     part = s - (item - p.split.first) * p.split.parts;
     parts = p.split.parts;
@@ -584,13 +593,25 @@ __global__ __attribute__((amdgpu_flat_work_group_size(256, 256), amdgpu_waves_pe
 hipError_t launch_bwd_dkdv64(BwdParams p, hipStream_t stream) {
   p.num_items = p.B * p.Hkv * (p.Skv / 128);
   // tail splitting (one work-group per compute unit); a part stores two 128 x 128 fp32 tiles
+  void* const caller_ws = p.split.ws;  // whether or not anything is split
   p.split = plan_split(p.num_items, 1, 2 * 128 * kHeadDim * 4, p.split.ws, p.split_ws_bytes);
   plan_xcd_mapping(p.B * p.Hkv, p.split.first, p.items_per_xcd, p.split.main_wgs);
   const int split_items = p.num_items - p.split.first;
   void (*fn)(const BwdParams) = p.ds_ws != nullptr ? &dkdv64_kernel<true> : &dkdv64_kernel<false>;
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(fn), hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes + 16);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(fn, dim3(p.split.main_wgs + split_items * p.split.parts), dim3(256), kSmemBytes, stream, p);
+  // Launches of several rounds with contiguous spans per XCD let the work-groups claim their grid indices, with some more
+  // work-groups than indices, so that an XCD that is through early takes over from the others (claim_work).
+  p.total_work = p.split.main_wgs + split_items * p.split.parts;
+  int grid = p.total_work;
+  p.queue = nullptr;
+  if (claims_wanted(p.items_per_xcd, p.total_work, 1))
+    p.queue = work_queue_in(caller_ws, p.split_ws_bytes, (int64_t)split_items * p.split.parts * 2 * 128 * kHeadDim * 4);
+  if (p.queue != nullptr) {
+    if ((e = launch_queue_reset(p.queue, stream)) != hipSuccess) return e;
+    grid += surplus_work_groups(p.total_work);
+  }
+  hipLaunchKernelGGL(fn, dim3(grid), dim3(256), kSmemBytes + 16, stream, p);
   if (split_items > 0) {
     const int64_t row0 = (int64_t)p.split.first * 128;
     e = launch_partial_sum(p.split.ws, p.split.parts, 2 * 128 * kHeadDim, p.dv, row0, split_items, 1.f, stream);

@@ -120,6 +120,23 @@ FBA_DEVICE float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 // measured 13-17 % slower).
 FBA_DEVICE int xcd_remap(int bid, int per_xcd) { return per_xcd > 0 ? (bid % kNumXcd) * per_xcd + bid / kNumXcd : bid; }
 
+// Work claimed instead of given.  The hardware deals work-groups to the eight XCDs round-robin, as many to a fast XCD as to
+// a slow one, and an XCD that is through with its share idles until the kernel ends.  A launch with a claim counter per XCD
+// (zeroed beforehand) has some work-groups more than grid indices to do; every work-group claims an index of its own XCD
+// (index = 8 k + XCD for the k-th claim there, so neighbours in the index space still meet in one L2) and, once those are
+// used up, of the other XCDs; a work-group that finds nothing left exits.  Returns -1 then.  One lane calls this.
+FBA_DEVICE int claim_work(int* counters, int xcd, int total) {
+  for (int d = 0; d < kNumXcd; ++d) {
+    const int y = (xcd + d) & (kNumXcd - 1);
+    const int k = atomicAdd(&counters[y], 1);
+    const int idx = kNumXcd * k + y;
+    if (idx < total) return idx;
+  }
+  return -1;
+}
+// XCD the wave runs on (0..7): XCC_ID field of the hardware register of that name.
+FBA_DEVICE int xcd_id() { return __builtin_amdgcn_s_getreg(20 | (3 << 11)) & (kNumXcd - 1); }
+
 // Cooperative copy of ROWS x 128 bf16 from global (row stride 256 B) into registers, then into a swizzled tile.
 // 256 threads; thread t owns chunk t % 16 of rows t / 16 + 16 i.
 template <int ROWS>

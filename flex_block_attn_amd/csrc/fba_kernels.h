@@ -103,6 +103,10 @@ struct BwdParams {
   const int32_t* k_slot;
   const char* zero_unit;
   SplitPlan split;
+  // dkdv64_kernel: claim counters, one per XCD, in the caller's tail-splitting workspace (null: work-group i does grid
+  // index i), and the number of grid indices there are to claim (see claim_work)
+  int* queue;
+  int total_work;
   int64_t split_ws_bytes;  // size of split.ws as handed in by the caller
 };
 
@@ -127,6 +131,16 @@ hipError_t launch_bwd_dq_from_ds(BwdParams p, hipStream_t stream);
 // once when they do not; this launch then fills `n` bf16 values at `out_a` (and at `out_b` unless null) with NaN, so that
 // the call fails loudly instead of writing out of bounds.
 hipError_t launch_poison_unless_fit(const BwdParams& p, __bf16* out_a, __bf16* out_b, int64_t n, hipStream_t stream);
+// Room for the claim counters behind `partial_bytes` of partial results in a tail-splitting workspace (null if there is
+// none), and the launch that zeroes them.
+int* work_queue_in(void* ws, int64_t ws_bytes, int64_t partial_bytes);
+// Is a launch of `total_work` grid indices at `wgs_per_cu` work-groups per compute unit worth claiming?  (At least four
+// rounds; FBA_CLAIM_WORK=0 in the environment switches claiming off, for measurements.)
+bool claims_wanted(int items_per_xcd, int total_work, int wgs_per_cu);
+// Work-groups launched on top of the grid indices of a claiming launch: an eighth more, a whole number per XCD.
+inline int surplus_work_groups(int total_work) { return (total_work / 8 + 7) / 8 * 8; }
+hipError_t launch_queue_reset(int* queue, hipStream_t stream);
+int device_compute_units();
 hipError_t launch_partial_sum(const float* ws, int parts, int64_t slot_floats, __bf16* out, int64_t out_row0, int n_items, float scale,
                               hipStream_t stream);
 hipError_t launch_probe_mfma(const float* src, float* sink, int work_groups, int iters, hipStream_t stream);

@@ -1,4 +1,5 @@
 // Tail splitting: which items of a launch are cut into parts (see SplitPlan in fba_kernels.h).
+#include <cstdlib>
 #include <mutex>
 
 #include "fba_kernels.h"
@@ -23,6 +24,32 @@ int compute_units() {
 }
 
 }  // namespace
+
+int device_compute_units() { return compute_units(); }
+
+namespace {
+constexpr int kQueueBytes = 256;
+__global__ void queue_reset_kernel(int* queue) { queue[threadIdx.x] = 0; }
+}  // namespace
+
+bool claims_wanted(int items_per_xcd, int total_work, int wgs_per_cu) {
+  const char* e = getenv("FBA_CLAIM_WORK");
+  const bool off = e != nullptr && e[0] == '0';
+  (void)items_per_xcd;  // either mapping deals grid index i to XCD i % 8, which is all a claim relies on
+  return !off && total_work >= 4 * compute_units() * wgs_per_cu;
+}
+
+int* work_queue_in(void* ws, int64_t ws_bytes, int64_t partial_bytes) {
+  if (ws == nullptr) return nullptr;
+  const int64_t off = (ws_bytes - kQueueBytes) & ~(int64_t)15;
+  if (off < partial_bytes) return nullptr;
+  return reinterpret_cast<int*>(static_cast<char*>(ws) + off);
+}
+
+hipError_t launch_queue_reset(int* queue, hipStream_t stream) {
+  hipLaunchKernelGGL(queue_reset_kernel, dim3(1), dim3(kQueueBytes / 4), 0, stream, queue);
+  return hipGetLastError();
+}
 
 // The hardware hands work-groups to free slots in index order.  With n items on s slots the last n % s items form a
 // partial round; when that round would fill at most half of the slots, each of its items is cut into floor(s / (n % s))

@@ -66,6 +66,11 @@ int32_t fba_mask_compact(const uint8_t* mask, int64_t mask_bh, int32_t nQ, int32
  *   split_ws_bytes  its size; fba_split_workspace_bytes() is what the planner can use at most (a smaller buffer limits
  *                   the number of ranges, never correctness)
  * On tile lists forward and the dK/dV kernel split; the dQ kernels do not.
+ * The same workspace lends its last 256 bytes (when they lie behind the partial results) to the dK/dV kernels of launches of
+ * four rounds and more: eight counters, zeroed by a one-wave launch in front, from which the work-groups claim the tile they
+ * work on, with an eighth more work-groups launched than there are tiles.  The hardware deals work-groups to the eight
+ * XCDs in equal numbers; with claims an XCD that is through with its share takes over tiles of the others instead of
+ * idling.  Which work-group computes a tile does not enter the result.
  */
 int64_t fba_split_workspace_bytes(void);
 

@@ -910,6 +910,31 @@ def test_handover_with_a_workspace_too_small_for_the_lists_fails_loudly(gpu, bs)
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("bs,keys", [(128, "64"), (128, "32"), (64, "32")])
+def test_claimed_grid_indices_change_no_bit(gpu, monkeypatch, bs, keys):
+    """Launches of four rounds and more let the dK/dV work-groups claim their grid indices (some work-groups more than
+    indices, an XCD that is through early takes over from the others): which work-group computes a tile must not show in
+    the result.  1152 key tiles; block lists with either dK/dV kernel, and tile lists."""
+    import flex_block_attn_amd as fba
+
+    B, H, S = 1, 9, 16384
+    g = torch.Generator(device="cpu").manual_seed(51 + bs)
+    q, k, v, do = (torch.randn((B, H, S, 128), generator=g).to(torch.bfloat16).to(gpu) for _ in range(4))
+    mask = (torch.rand((B, H, S // bs, S // bs), generator=g) < 0.1).to(gpu)
+    lists = fba.lists_for(mask, bs, bs)
+    o, lse = fba.forward_with_lists(q, k, v, bs, bs, lists)
+    monkeypatch.setenv("FBA_DKDV_KEYS_PER_WAVE", keys)
+    outs = []
+    for claim in ("0", None):
+        if claim is None:
+            monkeypatch.delenv("FBA_CLAIM_WORK", raising=False)
+        else:
+            monkeypatch.setenv("FBA_CLAIM_WORK", claim)
+        outs.append(fba.backward_with_lists(q, k, v, o, lse, do, bs, bs, lists))
+    for a, b in zip(*outs):
+        assert torch.isfinite(a).all() and torch.equal(a, b)
+
+
 def test_backward_memory_follows_the_sequence_length(gpu):
     """One head, S=30720, all 80 x 80 blocks of 384: the dS of that head (1.9 GB) is more than the default backward may
     allocate (six times the call's own tensors), so it recomputes instead and its peak allocation stays within twice the
