@@ -5,20 +5,21 @@ import torch
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("hand_over", [False, True])
-def test_step_replays_from_a_captured_graph(gpu, hand_over):
+@pytest.mark.parametrize("hand_over,shape", [(False, (4, 1536, 384)), (True, (4, 1536, 384)), (True, (9, 16384, 128))])
+def test_step_replays_from_a_captured_graph(gpu, hand_over, shape):
     """The library's launches record into a stream capture (no allocation, synchronisation or host read-back inside the
     C ABI), so a whole step on precompacted lists can be replayed as one graph.  Three replays with eager work and
     synchronisations in between, on fresh inputs written into the captured tensors, each compared bit for bit with the
-    eager result on the same inputs."""
+    eager result on the same inputs.  The third case is large enough (1152 key tiles) for the dK/dV work-groups to claim
+    their tiles from counters that a small launch inside the captured sequence zeroes on every replay."""
     import flex_block_attn_amd as fba
     from flex_block_attn_amd import interface, masks
 
-    B, H, S, bs = 1, 4, 1536, 384
+    B, (H, S, bs) = 1, shape
     g = torch.Generator(device="cpu").manual_seed(3)
     new = lambda: torch.randn((B, H, S, 128), generator=g).to(torch.bfloat16).to(gpu)
     q, k, v, do = new(), new(), new(), new()
-    mask = masks.random_block_mask(B, H, S // bs, S // bs, 2, seed=1).to(gpu)
+    mask = masks.random_block_mask(B, H, S // bs, S // bs, max(2, S // bs // 10), seed=1).to(gpu)
     lists = fba.compact_block_mask(mask, with_pair_numbers=True)
     lists.listed_pairs()  # the pair count reaches the host before the capture; nothing inside it waits
 
