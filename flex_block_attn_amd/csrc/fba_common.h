@@ -124,13 +124,24 @@ FBA_DEVICE int xcd_remap(int bid, int per_xcd) { return per_xcd > 0 ? (bid % kNu
 // a slow one, and an XCD that is through with its share idles until the kernel ends.  A launch with a claim counter per XCD
 // (zeroed beforehand) has some work-groups more than grid indices to do; every work-group claims an index of its own XCD
 // (index = 8 k + XCD for the k-th claim there, so neighbours in the index space still meet in one L2) and, once those are
-// used up, of the other XCDs; a work-group that finds nothing left exits.  Returns -1 then.  One lane calls this.
+// used up, of the XCD that has most left (all shares being equal, the one that has claimed least); a work-group that finds
+// nothing left exits.  Returns -1 then.  One lane calls this.
 FBA_DEVICE int claim_work(int* counters, int xcd, int total) {
-  for (int d = 0; d < kNumXcd; ++d) {
-    const int y = (xcd + d) & (kNumXcd - 1);
-    const int k = atomicAdd(&counters[y], 1);
-    const int idx = kNumXcd * k + y;
-    if (idx < total) return idx;
+  int k = atomicAdd(&counters[xcd], 1);
+  if (kNumXcd * k + xcd < total) return kNumXcd * k + xcd;
+  // own share used up: take from the XCD that has claimed least so far, i.e. has most left
+  for (int tries = 0; tries < kNumXcd; ++tries) {
+    int best = -1, least = 0x7fffffff;
+    for (int y = 0; y < kNumXcd; ++y) {
+      const int c = __atomic_load_n(&counters[y], __ATOMIC_RELAXED);
+      if (kNumXcd * c + y < total && c < least) {
+        least = c;
+        best = y;
+      }
+    }
+    if (best < 0) return -1;
+    k = atomicAdd(&counters[best], 1);
+    if (kNumXcd * k + best < total) return kNumXcd * k + best;
   }
   return -1;
 }
